@@ -1,0 +1,97 @@
+/* C ABI of libintra_hip.so: MI355X (gfx950) forward sparse-attention kernels of INTRA.
+ *
+ * This header is the drop-in boundary.  It replaces the pybind11 module `intra_attn_cuda` of the
+ * reference (csrc/flash_attn/flash_api.cpp:1766-1770, functions `fwd_llm` and `fwd`).  All tensor
+ * arguments are raw device pointers to bf16 data laid out (batch, token, head, 128) with the
+ * last dimension contiguous; strides are passed in ELEMENTS as {batch, token, head}.  Every
+ * pointer and every stride must keep 16-byte alignment (pointer % 16 == 0, stride % 8 == 0).
+ * The library allocates nothing and keeps no state between calls; the caller owns `o`.
+ * Launches are asynchronous on `hip_stream` (a hipStream_t, NULL = default stream).
+ *
+ * Every function returns INTRA_OK or an error code; intra_last_error() then describes the failure
+ * (thread-local string).  Argument validation happens before any HIP call, so it can be exercised
+ * on a machine without a GPU.
+ */
+#ifndef INTRA_HIP_H
+#define INTRA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  INTRA_OK = 0,
+  INTRA_ERR_INVALID = 1,     /* bad argument (null pointer, shape, stride, pattern id ...) */
+  INTRA_ERR_UNSUPPORTED = 2, /* valid request this build has no kernel for */
+  INTRA_ERR_HIP = 3          /* HIP runtime / launch failure */
+};
+
+/* Pattern ids, identical to the reference's `mask` argument
+ * (intra_attn/interface.py:12-13: LLM_PATTERNS, IMAGE_PATTERNS). */
+enum { INTRA_LLM_SCATTER = 0, INTRA_LLM_GATHER1 = 1, INTRA_LLM_WINDOW = 4 };
+enum { INTRA_IMAGE_SCATTER = 0, INTRA_IMAGE_GATHER0 = 4 };
+
+/* Causal language-model attention.  Replaces `fwd_llm` / mha_fwd_llm
+ * (csrc/flash_attn/flash_api.cpp:556-763) as called by intra_llm_attn
+ * (intra_attn/interface.py:30-45).
+ *   q, o: (B, S, H, 128); k, v: (B, S, Hkv, 128); H % Hkv == 0; query head h reads kv head
+ *   h / (H / Hkv).
+ *   pattern INTRA_LLM_SCATTER: group_num >= 1, any S.
+ *   pattern INTRA_LLM_GATHER1: group_num >= 1, any S (the reference is limited to 8 / S % 64 == 0).
+ *   pattern INTRA_LLM_WINDOW : window >= 64, any S; group_num ignored.
+ *   softmax_scale: any finite float. */
+int intra_llm_fwd(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                  int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                  int group_num, int window, float softmax_scale, void* hip_stream);
+
+/* Bidirectional attention over `text_len` text tokens followed by a width x width token grid.
+ * Replaces `fwd` / mha_fwd (csrc/flash_attn/flash_api.cpp:355-552) as called by intra_image_attn
+ * (intra_attn/interface.py:48-66).  S must equal text_len + width*width; width % 8 == 0,
+ * width >= 16, text_len % 8 == 0, text_len >= 8 (the reference fixes text_len = 512 and
+ * width in {64, 128}). */
+int intra_image_fwd(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                    int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                    const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                    int width, int text_len, float softmax_scale, void* hip_stream);
+
+/* Description of the last failure on the calling thread ("" if none).  Replaces the
+ * TORCH_CHECK messages of flash_api.cpp. */
+const char* intra_last_error(void);
+
+/* Library version, major*10000 + minor*100 + patch. */
+int intra_version(void);
+
+/* ------------------------------------------------------------------ host-only helpers (no GPU)
+ * How a call would be launched; mirrors the grid / per-set length derivation of the reference
+ * launchers (csrc/flash_attn/src/flash_fwd_launch_template.h:401-565, flash_api.cpp:408-411,
+ * 611-612, 703-714). */
+typedef struct IntraPlan {
+  int kind;            /* internal kernel kind 0..4 */
+  int heads_per_block; /* query heads of one kv head packed into a workgroup */
+  int waves;           /* wavefronts per workgroup */
+  int pos_per_block;   /* in-set queries per workgroup */
+  int n_sets;          /* sets per (batch, kv head) */
+  int n_mblocks;       /* row blocks of the largest set */
+  int grid;            /* workgroups launched */
+  int lds_bytes;       /* LDS per workgroup */
+  int64_t pairs_per_head; /* unmasked (query, key) pairs per query head and batch */
+} IntraPlan;
+
+/* domain 0 = LLM (arg0 = group_num, arg1 = window), 1 = image (arg0 = width, arg1 = text_len). */
+int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
+               IntraPlan* plan);
+
+/* Walks the exact set / row-block / wavefront / 32-key-block decomposition the kernel uses
+ * (same index maps and block classification, compiled for the host) and adds 1 to
+ * count[q_pos * S + k_pos] for every score the kernel would compute and keep.  `count` is an
+ * S*S byte array the caller zeroed.  heads_per_block / waves <= 0 pick the library default. */
+int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int heads_per_block,
+                     int waves, uint8_t* count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INTRA_HIP_H */

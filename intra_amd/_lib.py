@@ -1,0 +1,57 @@
+"""ctypes binding of libintra_hip.so (declared in include/intra_hip.h)."""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libintra_hip.so")
+
+INTRA_OK, INTRA_ERR_INVALID, INTRA_ERR_UNSUPPORTED, INTRA_ERR_HIP = 0, 1, 2, 3
+
+_i64x3 = ctypes.c_int64 * 3
+
+
+class IntraPlan(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int), ("heads_per_block", ctypes.c_int), ("waves", ctypes.c_int),
+                ("pos_per_block", ctypes.c_int), ("n_sets", ctypes.c_int), ("n_mblocks", ctypes.c_int),
+                ("grid", ctypes.c_int), ("lds_bytes", ctypes.c_int), ("pairs_per_head", ctypes.c_int64)]
+
+
+_FWD_ARGS = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 4 + \
+    [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_float, ctypes.c_void_p]
+
+SYMBOLS = {
+    "intra_llm_fwd": (ctypes.c_int, _FWD_ARGS),
+    "intra_image_fwd": (ctypes.c_int, _FWD_ARGS),
+    "intra_last_error": (ctypes.c_char_p, []),
+    "intra_version": (ctypes.c_int, []),
+    "intra_plan": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.POINTER(IntraPlan)]),
+    "intra_model_mask": (ctypes.c_int, [ctypes.c_int] * 7 + [ctypes.c_void_p]),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library once.  Raises ImportError if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(f"{LIB_PATH} is not built; run `python -m intra_amd.build`")
+        try:
+            lib = ctypes.CDLL(LIB_PATH)
+        except OSError as err:
+            raise ImportError(f"cannot load {LIB_PATH}: {err}") from err
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def last_error():
+    return load().intra_last_error().decode()
+
+
+def strides3(x):
+    """(batch, token, head) element strides of a (B, S, H, D) tensor as a C array."""
+    return _i64x3(x.stride(0), x.stride(1), x.stride(2))

@@ -1,0 +1,46 @@
+"""Builds libintra_hip.so for gfx950 with hipcc (no torch or CUDA-compat headers involved).
+
+    python -m intra_amd.build
+
+Takes the place of the reference's CUDAExtension build (setup.py:28-68).
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+SRC = os.path.join(HERE, "csrc", "intra_api.hip")
+LIB = os.path.join(HERE, "libintra_hip.so")
+
+# -packed-fp32-ops off: plain v_add/v_mul/v_fma only, no v_pk_*_f32 forms.
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-shared", "-fPIC",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def hipcc_path():
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found; set HIPCC or install ROCm")
+
+
+def build(verbose=False, extra_flags=()):
+    """Compile the library in-tree and return its path."""
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, SRC, "-o", LIB + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "not a recognized feature" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
+    if verbose and out.strip():
+        print(out)
+    os.replace(LIB + ".tmp", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True, extra_flags=sys.argv[1:]))

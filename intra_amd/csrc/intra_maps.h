@@ -1,0 +1,196 @@
+// Computational Query Set (CQS) index maps and key bounds, shared by the gfx950 kernels and by
+// the host-side model that the CPU tests walk.
+//
+// A "set" is a group of query tokens that share one packed key list.  Inside a set, queries are
+// numbered tq = 0..nq-1 and keys tk = 0..nk-1 ("in-set indices"); qpos()/kpos() turn an in-set
+// index into a token position of the (B, S, H, 128) tensors.  Query tq attends exactly the keys
+// klo(tq) <= tk <= min(khi(tq), nk-1).  klo and khi are non-decreasing in tq for every pattern,
+// which is what lets a wavefront classify a whole 32x32 score block as skipped / unmasked /
+// partially masked from the bounds of its first and last query alone.
+//
+// Semantics follow the dense-mask specification of the reference:
+//   LLM scatter   intra_attn/reference.py:14-17    index map csrc/flash_attn/src/gmem_tile.h:511,656
+//   LLM gather1   intra_attn/reference.py:20-24    gmem_tile.h:847-864
+//   LLM window    intra_attn/reference.py:27-32    csrc/flash_attn/src/flash_fwd_kernel.h:7008
+//   image scatter intra_attn/reference.py:36-53    gmem_tile.h:286-340,388-389
+//   image gather0 intra_attn/reference.py:56-74    gmem_tile.h:1220-1294,1334-1373
+// The maps here are re-derived from those predicates; nothing is shared with the reference code.
+#pragma once
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define IM_HD __host__ __device__ __forceinline__
+#else
+#define IM_HD inline
+#endif
+
+// Pattern kinds used inside the library (the public pattern ids are per-entry-point).
+enum IntraKind : int {
+  KIND_LLM_SCATTER = 0,
+  KIND_LLM_GATHER1 = 1,
+  KIND_LLM_WINDOW = 2,
+  KIND_IMG_SCATTER = 3,
+  KIND_IMG_GATHER0 = 4,
+};
+
+struct IntraGeom {
+  int S;         // tokens per sequence
+  int G;         // LLM scatter / gather1 group count
+  int window;    // LLM window width in keys (>= 64)
+  int width;     // image latent grid side (tokens)
+  int text_len;  // image: text tokens in front of the grid
+};
+
+IM_HD int im_min(int a, int b) { return a < b ? a : b; }
+IM_HD int im_max(int a, int b) { return a > b ? a : b; }
+
+// ---------------------------------------------------------------- LLM scatter: token i in group i % G
+struct MapLlmScatter {
+  int G, g, n;
+  static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
+  static IM_HD int max_nq(const IntraGeom& ge) { return (ge.S + ge.G - 1) / ge.G; }
+  IM_HD MapLlmScatter(const IntraGeom& ge, int set) {
+    G = ge.G;
+    g = set;
+    n = ge.S > set ? (ge.S - set + ge.G - 1) / ge.G : 0;
+  }
+  IM_HD int nq() const { return n; }
+  IM_HD int nk() const { return n; }
+  IM_HD int qpos(int t) const { return t * G + g; }
+  IM_HD int kpos(int t) const { return t * G + g; }
+  IM_HD int klo(int) const { return 0; }
+  IM_HD int khi(int tq) const { return tq; }
+};
+
+// ------------------------------------- LLM gather1: segments of G tokens, segment s in group s % G
+// Token p = (G*G)*a + G*g + r (r < G) is in-set index G*a + r of group g; positions grow with the
+// in-set index, so causality in positions equals causality in in-set indices.
+struct MapLlmGather1 {
+  int G, g, n;
+  static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
+  static IM_HD int max_nq(const IntraGeom& ge) {
+    int gg = ge.G * ge.G;
+    return (ge.S / gg) * ge.G + im_min(ge.G, ge.S % gg);
+  }
+  IM_HD MapLlmGather1(const IntraGeom& ge, int set) {
+    G = ge.G;
+    g = set;
+    int gg = G * G;
+    int rem = ge.S % gg - G * g;  // tokens of this group in the last, partial G*G block
+    n = (ge.S / gg) * G + im_max(0, im_min(G, rem));
+  }
+  IM_HD int nq() const { return n; }
+  IM_HD int nk() const { return n; }
+  IM_HD int qpos(int t) const { return (t / G) * (G * G) + g * G + t % G; }
+  IM_HD int kpos(int t) const { return qpos(t); }
+  IM_HD int klo(int) const { return 0; }
+  IM_HD int khi(int tq) const { return tq; }
+};
+
+// -------------------------- LLM window: 64-query blocks see themselves plus window-64 earlier tokens
+struct MapLlmWindow {
+  int S, lookback;
+  static IM_HD int num_sets(const IntraGeom&) { return 1; }
+  static IM_HD int max_nq(const IntraGeom& ge) { return ge.S; }
+  IM_HD MapLlmWindow(const IntraGeom& ge, int) {
+    S = ge.S;
+    lookback = ge.window - 64;
+  }
+  IM_HD int nq() const { return S; }
+  IM_HD int nk() const { return S; }
+  IM_HD int qpos(int t) const { return t; }
+  IM_HD int kpos(int t) const { return t; }
+  IM_HD int klo(int tq) const { return im_max((tq & ~63) - lookback, 0); }
+  IM_HD int khi(int tq) const { return tq; }
+};
+
+// ------------- image scatter: 8 groups, grid token (r, c) in group (r%2)*4 + c%4, text chunk j rides
+// with group j; every query sees all text keys plus the grid keys of its own group.
+struct MapImgScatter {
+  int W, T, chunk, j, a, b, wq, nimg;
+  static IM_HD int num_sets(const IntraGeom&) { return 8; }
+  static IM_HD int max_nq(const IntraGeom& ge) { return ge.text_len / 8 + ge.width * ge.width / 8; }
+  IM_HD MapImgScatter(const IntraGeom& ge, int set) {
+    W = ge.width;
+    T = ge.text_len;
+    chunk = T / 8;
+    j = set;
+    a = set >> 2;
+    b = set & 3;
+    wq = W / 4;
+    nimg = W * W / 8;
+  }
+  IM_HD int imgpos(int u) const { return T + (a + 2 * (u / wq)) * W + b + 4 * (u % wq); }
+  IM_HD int nq() const { return chunk + nimg; }
+  IM_HD int nk() const { return T + nimg; }
+  IM_HD int qpos(int t) const { return t < chunk ? chunk * j + t : imgpos(t - chunk); }
+  IM_HD int kpos(int t) const { return t < T ? t : imgpos(t - T); }
+  IM_HD int klo(int) const { return 0; }
+  IM_HD int khi(int) const { return T + nimg - 1; }
+};
+
+// ---- image gather0: every 8x8 patch of grid queries sees all text plus a 16x16 grid window around
+// it (shifted inwards at the borders); text queries keep their scatter rows.  Sets 0..7 are the text
+// chunks (keys = scatter key list of group j), sets 8.. are the patches in row-major patch order.
+struct MapImgGather0 {
+  int W, T, chunk, m, r0, c0, qr, qc;
+  MapImgScatter sc;
+  static IM_HD int num_sets(const IntraGeom& ge) { return 8 + (ge.width / 8) * (ge.width / 8); }
+  static IM_HD int max_nq(const IntraGeom& ge) { return im_max(ge.text_len / 8, 64); }
+  static IM_HD int win_start(int idx, int np) {
+    if (idx == np - 1) return idx * 8 - 8;
+    if (idx == 0) return 0;
+    return idx * 8 - 4;
+  }
+  IM_HD MapImgGather0(const IntraGeom& ge, int set) : sc(ge, set < 8 ? set : 0) {
+    W = ge.width;
+    T = ge.text_len;
+    chunk = T / 8;
+    m = set;
+    int np = W / 8;
+    int P = set < 8 ? 0 : set - 8;
+    int R = P / np, C = P % np;
+    qr = 8 * R;
+    qc = 8 * C;
+    r0 = win_start(R, np);
+    c0 = win_start(C, np);
+  }
+  IM_HD int nq() const { return m < 8 ? chunk : 64; }
+  IM_HD int nk() const { return m < 8 ? sc.nk() : T + 256; }
+  IM_HD int qpos(int t) const { return m < 8 ? chunk * m + t : T + (qr + (t >> 3)) * W + qc + (t & 7); }
+  IM_HD int kpos(int t) const {
+    if (m < 8) return sc.kpos(t);
+    if (t < T) return t;
+    int u = t - T;
+    return T + (r0 + (u >> 4)) * W + c0 + (u & 15);
+  }
+  IM_HD int klo(int) const { return 0; }
+  IM_HD int khi(int) const { return nk() - 1; }
+};
+
+// --------------------------------------------------------------------------- tile classification
+// A wavefront owns the queries wq0..wq_last of a set and looks at the 32 keys sb_lo..sb_lo+31.
+enum : int { BLK_SKIP = 0, BLK_FULL = 1, BLK_PARTIAL = 2 };
+
+struct WaveBounds {
+  int w_lo, w_hi;  // union of the key ranges of the wavefront's queries
+  int f_lo, f_hi;  // intersection of them
+};
+
+template <class MAP>
+IM_HD WaveBounds wave_bounds(const MAP& map, int wq0, int wq_last) {
+  int kmax = map.nk() - 1;
+  WaveBounds wb;
+  wb.w_lo = map.klo(wq0);
+  wb.w_hi = im_min(map.khi(wq_last), kmax);
+  wb.f_lo = map.klo(wq_last);
+  wb.f_hi = im_min(map.khi(wq0), kmax);
+  return wb;
+}
+
+IM_HD int classify_block(const WaveBounds& wb, int sb_lo) {
+  int sb_hi = sb_lo + 31;
+  if (sb_lo > wb.w_hi || sb_hi < wb.w_lo) return BLK_SKIP;
+  if (sb_lo >= wb.f_lo && sb_hi <= wb.f_hi) return BLK_FULL;
+  return BLK_PARTIAL;
+}

@@ -1,0 +1,95 @@
+"""Python entry points of the MI355X INTRA kernels (forward only).
+
+Same surface as the reference's intra_attn/interface.py:12-66: `intra_llm_attn` and
+`intra_image_attn` take q, k, v of shape (batch, seqlen, heads, 128) in bfloat16 on the GPU and
+return the attention output in q's layout; k/v may have fewer heads than q (GQA) as long as they
+divide the query heads.  Pattern names, arguments, defaults and exception types are the
+reference's.  The work is done by libintra_hip.so through its C ABI (include/intra_hip.h); there
+is no fallback path, a missing library is an ImportError.
+"""
+import torch
+
+from . import _lib
+
+_C = _lib.load()
+
+LLM_PATTERNS = {"scatter": 0, "gather1": 1, "window": 4}
+IMAGE_PATTERNS = {"scatter": 0, "gather0": 4}
+TEXT_LEN = 512
+
+
+def _aligned(x):
+    return x.stride(-1) == 1 and x.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in x.stride()[:-1])
+
+
+def _check(q, k, v):
+    # reference: intra_attn/interface.py:17-23 (same conditions, same exception types and texts)
+    for x in (q, k, v):
+        if not x.is_cuda or x.dtype != torch.bfloat16 or x.shape[-1] != 128:
+            raise ValueError("INTRA kernels need CUDA bfloat16 tensors with head_dim 128")
+    if torch.is_grad_enabled() and any(x.requires_grad for x in (q, k, v)):
+        raise RuntimeError("INTRA kernels are forward-only; call them under torch.no_grad()")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise ValueError("q, k, v must be (batch, seqlen, heads, 128)")
+    if k.shape != v.shape or k.shape[:2] != q.shape[:2] or q.shape[2] % k.shape[2]:
+        raise RuntimeError(f"q {tuple(q.shape)} and k/v {tuple(k.shape)}/{tuple(v.shape)} do not "
+                           "match: need equal batch and seqlen, and query heads divisible by kv heads")
+    # The kernels honour arbitrary batch/token/head strides; only rows that are not contiguous
+    # or not 16-byte aligned are copied.
+    return [x if _aligned(x) else x.contiguous() for x in (q, k, v)]
+
+
+def _scale(q, softmax_scale):
+    return q.shape[-1] ** -0.5 if softmax_scale is None else softmax_scale
+
+
+def _launch(fn, q, k, v, pattern_id, arg0, arg1, scale):
+    out = torch.empty_like(q)
+    if not _aligned(out):
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    B, S, H, _ = q.shape
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
+                _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                pattern_id, arg0, arg1, float(scale), stream)
+    if rc != _lib.INTRA_OK:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
+    return out
+
+
+def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None):
+    """Causal prefill attention for language models.
+
+    pattern="scatter": token i attends to earlier tokens j with j % group_num == i % group_num.
+    pattern="gather1": groups are segments of group_num tokens, segment s in group s % group_num.
+    pattern="window":  each 64-query block attends to itself and the preceding window - 64 tokens.
+
+    Any seqlen works for scatter and window; gather1 keeps the reference's contract of
+    group_num=8 and seqlen % 64 == 0 (intra_attn/interface.py:41-42).
+    """
+    q, k, v = _check(q, k, v)
+    if pattern == "gather1" and (group_num != 8 or q.shape[1] % (group_num * group_num)):
+        raise ValueError(f"gather1 needs group_num=8 and seqlen % 64 == 0, got G={group_num}, S={q.shape[1]}")
+    return _launch(_C.intra_llm_fwd, q, k, v, LLM_PATTERNS[pattern], int(group_num), int(window),
+                   _scale(q, softmax_scale))
+
+
+def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None):
+    """Bidirectional attention for FLUX-style sequences: 512 text tokens followed by a
+    width x width grid of image tokens.
+
+    pattern="scatter": 8 groups, image token (r, c) in group (r % 2) * 4 + c % 4; text chunks of
+                       64 tokens ride with groups 0..7; all text keys are always visible.
+    pattern="gather0": each 8 x 8 image patch attends to a 16 x 16 window around it plus all text.
+
+    Width 64 (1024 x 1024 FLUX images) and 128 (2048 x 2048), as in the reference
+    (intra_attn/interface.py:59-63).
+    """
+    q, k, v = _check(q, k, v)
+    if width not in (64, 128):
+        raise ValueError("image kernels are compiled for width 64 and 128")
+    if q.shape[1] != TEXT_LEN + width * width:
+        raise ValueError(f"expected {TEXT_LEN} text + {width}x{width} image tokens, got {q.shape[1]}")
+    return _launch(_C.intra_image_fwd, q, k, v, IMAGE_PATTERNS[pattern], int(width), TEXT_LEN,
+                   _scale(q, softmax_scale))

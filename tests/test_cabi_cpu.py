@@ -1,0 +1,133 @@
+"""CPU-side checks of libintra_hip.so: it loads, exports every symbol of include/intra_hip.h,
+validates arguments without touching a GPU, plans launches, and its host walk of the kernel's
+set / row-block / wavefront / key-block decomposition reproduces the oracle masks exactly."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from intra_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_exports_every_declared_symbol(lib):
+    header = open(os.path.join(ROOT, "include", "intra_hip.h")).read()
+    declared = set(re.findall(r"^\s*(?:const\s+char\*|int)\s+(intra_\w+)\s*\(", header, re.M))
+    assert declared == set(_lib.SYMBOLS), (declared, set(_lib.SYMBOLS))
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.intra_version() >= 100
+
+
+def _plan(lib, domain, pattern, B, S, H, Hkv, a0, a1):
+    p = _lib.IntraPlan()
+    rc = lib.intra_plan(domain, pattern, B, S, H, Hkv, a0, a1, ctypes.byref(p))
+    return rc, p
+
+
+def test_plan_headline(lib):
+    rc, p = _plan(lib, 0, 0, 1, 32768, 32, 8, 8, 576)
+    assert rc == 0
+    assert (p.heads_per_block, p.waves, p.pos_per_block) == (4, 8, 64)
+    assert (p.n_sets, p.n_mblocks, p.grid) == (8, 64, 4096)
+    assert p.pairs_per_head == 67125248 and p.lds_bytes == 65536
+
+
+@pytest.mark.parametrize("domain,pattern,kind,S,a0,a1", [
+    (0, 0, "llm/scatter", 1000, 3, 576), (0, 1, "llm/gather1", 3000, 8, 576),
+    (0, 4, "llm/window", 3000, 8, 1000), (1, 0, "image/scatter", 4608, 64, 512),
+    (1, 4, "image/gather0", 16896, 128, 512)])
+def test_plan_pair_counts(lib, domain, pattern, kind, S, a0, a1):
+    rc, p = _plan(lib, domain, pattern, 1, S, 8, 8, a0, a1)
+    assert rc == 0
+    kw = dict(group_num=a0, window=a1) if domain == 0 else dict(width=a0, text_len=a1)
+    assert p.pairs_per_head == oracle.pairs_per_head(kind, S, **kw)
+
+
+BAD = [  # domain, pattern, B, S, H, Hkv, a0, a1, text in the message
+    (0, 7, 1, 128, 4, 4, 8, 576, "unknown LLM pattern"),
+    (0, 0, 1, 128, 4, 3, 8, 576, "multiple of kv heads"),
+    (0, 0, 0, 128, 4, 4, 8, 576, "must be positive"),
+    (0, 0, 1, 128, 4, 4, 0, 576, "group_num must be >= 1"),
+    (0, 4, 1, 128, 4, 4, 8, 32, "window must be >= 64"),
+    (1, 1, 1, 4608, 4, 4, 64, 512, "unknown image pattern"),
+    (1, 0, 1, 4600, 4, 4, 64, 512, "expected 512 text + 64x64"),
+    (1, 0, 1, 512 + 100, 4, 4, 10, 512, "width must be a multiple of 8"),
+    (1, 4, 1, 500 + 4096, 4, 4, 64, 500, "text_len must be a positive multiple of 8"),
+    (2, 0, 1, 128, 4, 4, 8, 576, "unknown domain"),
+]
+
+
+@pytest.mark.parametrize("case", BAD)
+def test_plan_rejects_bad_requests(lib, case):
+    *args, text = case
+    rc, _ = _plan(lib, *args)
+    assert rc == _lib.INTRA_ERR_INVALID
+    assert text in _lib.last_error()
+
+
+def test_fwd_validates_before_touching_the_gpu(lib):
+    st = (ctypes.c_int64 * 3)(128 * 4 * 128, 4 * 128, 128)
+    bad = (ctypes.c_int64 * 3)(128 * 4 * 128, 4 * 128 + 4, 128)
+    ptr = 1 << 20  # never dereferenced: every call below fails validation first
+    call = lambda *a: lib.intra_llm_fwd(*a)
+    assert call(None, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, st, 0, 8, 576, 0.1, None) == 1
+    assert "non-null" in _lib.last_error()
+    assert call(ptr + 2, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, st, 0, 8, 576, 0.1, None) == 1
+    assert "16-byte aligned" in _lib.last_error()
+    assert call(ptr, ptr, ptr, ptr, 1, 128, 4, 4, st, bad, st, st, 0, 8, 576, 0.1, None) == 1
+    assert "k stride 1" in _lib.last_error()
+    assert call(ptr, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, None, 0, 8, 576, 0.1, None) == 1
+    assert "o strides pointer is null" in _lib.last_error()
+    assert call(ptr, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, st, 0, 8, 576, float("nan"), None) == 1
+    assert "finite" in _lib.last_error()
+    assert call(ptr, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, st, 9, 8, 576, 0.1, None) == 1
+    assert lib.intra_image_fwd(ptr, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, st, 0, 64, 512, 0.1, None) == 1
+    assert "expected 512 text" in _lib.last_error()
+
+
+def _model(lib, domain, pattern, S, a0, a1, hp=0, nw=0):
+    count = np.zeros((S, S), dtype=np.uint8)
+    rc = lib.intra_model_mask(domain, pattern, S, a0, a1, hp, nw, count.ctypes.data)
+    assert rc == 0, _lib.last_error()
+    return torch.from_numpy(count)
+
+
+LLM_CASES = [(S, "llm/scatter", 0, dict(group_num=G)) for S in (1, 5, 63, 64, 65, 257, 1000) for G in (1, 2, 3, 8, 16)] + \
+            [(S, "llm/gather1", 1, dict(group_num=G)) for S in (64, 128, 1000, 1024) for G in (8, 3)] + \
+            [(S, "llm/window", 4, dict(window=W)) for S in (1, 64, 100, 1000, 1300) for W in (64, 65, 96, 576, 1000, 5000)]
+
+
+@pytest.mark.parametrize("S,kind,pattern,kw", LLM_CASES)
+@pytest.mark.parametrize("hp", [1, 2, 4])
+def test_kernel_decomposition_equals_mask_llm(lib, S, kind, pattern, kw, hp):
+    count = _model(lib, 0, pattern, S, kw.get("group_num", 8), kw.get("window", 576), hp, 8)
+    want = oracle.mask_rows(kind, S, **kw)
+    assert count.max() <= 1, "a score is computed more than once"
+    assert torch.equal(count.bool(), want)
+
+
+IMG_CASES = [(16, 64), (24, 16), (32, 512), (64, 512), (40, 8)]
+
+
+@pytest.mark.parametrize("W,T", IMG_CASES)
+@pytest.mark.parametrize("kind,pattern", [("image/scatter", 0), ("image/gather0", 4)])
+@pytest.mark.parametrize("hp", [1, 2, 4])
+def test_kernel_decomposition_equals_mask_image(lib, W, T, kind, pattern, hp):
+    S = T + W * W
+    nw = 2 * hp if pattern == 4 else 8
+    count = _model(lib, 1, pattern, S, W, T, hp, nw)
+    want = oracle.mask_rows(kind, S, width=W, text_len=T)
+    assert count.max() <= 1
+    assert torch.equal(count.bool(), want)
+
+
+def test_model_rejects_unknown_shape(lib):
+    count = np.zeros((64, 64), dtype=np.uint8)
+    assert lib.intra_model_mask(0, 0, 64, 8, 576, 3, 8, count.ctypes.data) == 1
+    assert "no kernel" in _lib.last_error()

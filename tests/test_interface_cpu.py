@@ -1,0 +1,40 @@
+"""Error contract of the Python API on a machine without a GPU (intra_attn/interface.py:17-23,
+41-42, 60-63 of the reference): the checks fire before anything is launched."""
+import pytest
+import torch
+
+import intra_amd
+import intra_attn
+from intra_amd import interface
+
+
+def _cpu(S=128, H=4, Hkv=4, dtype=torch.bfloat16, D=128):
+    return (torch.zeros(1, S, H, D, dtype=dtype), torch.zeros(1, S, Hkv, D, dtype=dtype),
+            torch.zeros(1, S, Hkv, D, dtype=dtype))
+
+
+def test_names_and_constants():
+    assert intra_attn.intra_llm_attn is intra_amd.intra_llm_attn
+    assert intra_attn.intra_image_attn is intra_amd.intra_image_attn
+    assert interface.LLM_PATTERNS == {"scatter": 0, "gather1": 1, "window": 4}
+    assert interface.IMAGE_PATTERNS == {"scatter": 0, "gather0": 4}
+    assert interface.TEXT_LEN == 512 and intra_amd.__version__
+
+
+def test_signatures_match_reference():
+    import inspect
+    llm = inspect.signature(intra_amd.intra_llm_attn)
+    assert list(llm.parameters) == ["q", "k", "v", "pattern", "group_num", "window", "softmax_scale"]
+    assert [p.default for p in llm.parameters.values()][3:] == ["scatter", 8, 576, None]
+    img = inspect.signature(intra_amd.intra_image_attn)
+    assert list(img.parameters) == ["q", "k", "v", "pattern", "width", "softmax_scale"]
+    assert [p.default for p in img.parameters.values()][3:] == ["scatter", 64, None]
+
+
+@pytest.mark.parametrize("make", [lambda: _cpu(), lambda: _cpu(dtype=torch.float16), lambda: _cpu(D=64)])
+def test_rejects_non_cuda_bf16_128(make):
+    q, k, v = make()
+    with pytest.raises(ValueError, match="CUDA bfloat16 tensors with head_dim 128"):
+        intra_amd.intra_llm_attn(q, k, v)
+    with pytest.raises(ValueError, match="CUDA bfloat16 tensors with head_dim 128"):
+        intra_amd.intra_image_attn(q, k, v)

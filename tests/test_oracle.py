@@ -1,0 +1,233 @@
+"""Pins the CPU oracle (oracle/) without the reference on the path.
+
+Each check is independent of the oracle's own formulas: loop constructions written from the
+prose description of a pattern, the known answers and invariants that the reference's self-check
+holds (intra_attn/reference.py:86-103), the mask densities its FLUX mask test prints
+(experiments/flux/test_masks.py:126-134: 22.2 % / 17.3 %), a float64 triple loop, and torch's
+scaled_dot_product_attention, which is the library routine the reference's oracle consists of.
+"""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from oracle import masks, pairs
+
+
+# ------------------------------------------------------------------ LLM masks
+@pytest.mark.parametrize("S,G", [(32, 4), (37, 3), (64, 8), (100, 8), (5, 8), (50, 1), (33, 2)])
+def test_llm_scatter_bruteforce(S, G):
+    m = masks.llm_scatter_mask(S, G)
+    for a in range(S):
+        for b in range(S):
+            assert bool(m[a, b]) == (b <= a and a % G == b % G)
+
+
+@pytest.mark.parametrize("S,G", [(32, 4), (128, 8), (64, 8), (70, 3), (200, 8)])
+def test_llm_gather1_bruteforce(S, G):
+    m = masks.llm_gather1_mask(S, G)
+    for a in range(S):
+        for b in range(S):
+            assert bool(m[a, b]) == (b <= a and (a // G) % G == (b // G) % G)
+
+
+def test_llm_gather1_by_segments():
+    # built from the prose: cut the sequence into segments of G tokens, deal segments to groups
+    # round-robin, attend causally inside a group
+    S, G = 256, 8
+    group_of = []
+    for seg in range(math.ceil(S / G)):
+        group_of += [seg % G] * G
+    m = masks.llm_gather1_mask(S, G)
+    for a in range(S):
+        for b in range(S):
+            assert bool(m[a, b]) == (b <= a and group_of[a] == group_of[b])
+
+
+def test_llm_window_known_answers():
+    # reference.py:93-94
+    m = masks.llm_window_mask(200, window=96, block=64)
+    assert m[130, 128 - 32] and not m[130, 128 - 33] and m[63, 0] and not m[10, 11]
+
+
+@pytest.mark.parametrize("S,W", [(200, 96), (1000, 576), (700, 64), (300, 1000), (640, 130)])
+def test_llm_window_by_blocks(S, W):
+    # prose: a block of 64 queries sees itself (causally) and the W - 64 tokens before the block
+    want = torch.zeros(S, S, dtype=torch.bool)
+    for b0 in range(0, S, 64):
+        first = max(b0 - (W - 64), 0)
+        for i in range(b0, min(b0 + 64, S)):
+            want[i, first:i + 1] = True
+    assert torch.equal(masks.llm_window_mask(S, W), want)
+
+
+def test_llm_window_key_counts():
+    # rows far enough in see between W-63 and W keys
+    S, W = 4096, 576
+    cnt = masks.llm_window_mask(S, W).sum(1)
+    assert cnt[W:].min() == W - 63 and cnt.max() == W
+    assert cnt[0] == 1 and cnt[63] == 64
+
+
+# ------------------------------------------------------------------ image masks
+def _loop_image_scatter(W, T):
+    S = T + W * W
+    grp = [t // (T // 8) for t in range(T)]
+    for r in range(W):
+        for c in range(W):
+            grp.append((r % 2) * 4 + c % 4)
+    want = torch.zeros(S, S, dtype=torch.bool)
+    members = [[p for p in range(T, S) if grp[p] == g] for g in range(8)]
+    for i in range(S):
+        want[i, :T] = True
+        want[i, members[grp[i]]] = True
+    return want
+
+
+def _loop_image_gather0(W, T):
+    S = T + W * W
+    want = _loop_image_scatter(W, T)
+    n = W // 8
+    for R in range(n):
+        for C in range(n):
+            def first(idx):
+                if idx == 0:
+                    return 0
+                if idx == n - 1:
+                    return 8 * idx - 8
+                return 8 * idx - 4
+            r0, c0 = first(R), first(C)
+            keys = [T + r * W + c for r in range(r0, r0 + 16) for c in range(c0, c0 + 16)]
+            for r in range(8 * R, 8 * R + 8):
+                for c in range(8 * C, 8 * C + 8):
+                    i = T + r * W + c
+                    want[i] = False
+                    want[i, :T] = True
+                    want[i, keys] = True
+    return want
+
+
+@pytest.mark.parametrize("W,T", [(16, 64), (32, 512), (24, 16)])
+def test_image_masks_by_loops_small(W, T):
+    assert torch.equal(masks.image_scatter_mask(W, T), _loop_image_scatter(W, T))
+    assert torch.equal(masks.image_gather0_mask(W, T), _loop_image_gather0(W, T))
+
+
+def test_image_masks_by_loops_flux_1024():
+    assert torch.equal(masks.image_scatter_mask(64), _loop_image_scatter(64, 512))
+    assert torch.equal(masks.image_gather0_mask(64), _loop_image_gather0(64, 512))
+
+
+def test_image_invariants_reference_selfcheck():
+    # reference.py:95-102
+    W, T = 64, masks.TEXT_LEN
+    m = masks.image_scatter_mask(W)
+    assert m.shape == (T + W * W,) * 2 and m[:, :T].all()
+    assert m[T:, T:].sum(1).eq(W * W // 8).all()
+    m = masks.image_gather0_mask(W)
+    assert m[T:, T:].sum(1).eq(256).all()
+    q = T + 9 * W + 9  # patch (1, 1) -> window rows/cols 4..19
+    assert m[q, T + 4 * W + 4] and not m[q, T + 3 * W + 4] and m[q, T + 19 * W + 19]
+    assert not m[q, T + 20 * W + 19] and not m[q, T + 4 * W + 3]
+
+
+def test_image_densities_published():
+    # experiments/flux/test_masks.py prints density 0.2222 (scatter) and 0.1728 (gather0) at W=64
+    assert abs(masks.image_scatter_mask(64).float().mean().item() - 0.2222) < 5e-5
+    assert abs(masks.image_gather0_mask(64).float().mean().item() - 0.1728) < 5e-5
+
+
+def test_image_w128_invariants():
+    W, T = 128, 512
+    rows = torch.cat([torch.arange(0, T, 37), T + torch.arange(0, W * W, 251)])
+    ms = masks.image_scatter_mask(W, rows=rows)
+    assert ms[:, :T].all() and ms[:, T:].sum(1).eq(W * W // 8).all()
+    mg = masks.image_gather0_mask(W, rows=rows)
+    is_text = rows < T
+    assert mg[is_text][:, T:].sum(1).eq(W * W // 8).all()
+    assert mg[~is_text][:, T:].sum(1).eq(256).all()
+    # last patch (15, 15): window rows/cols 112..127
+    q = T + 127 * W + 127
+    row = masks.image_gather0_mask(W, rows=torch.tensor([q]))[0]
+    assert row[T + 112 * W + 112] and not row[T + 111 * W + 112] and row[T + 127 * W + 127]
+
+
+@pytest.mark.parametrize("kind,S,kw", [
+    ("llm/scatter", 1000, dict(group_num=3)), ("llm/gather1", 1024, dict(group_num=8)),
+    ("llm/window", 1000, dict(window=576)), ("image/scatter", 64 + 256, dict(width=16, text_len=64)),
+    ("image/gather0", 512 + 1024, dict(width=32))])
+def test_row_subset_equals_full(kind, S, kw):
+    full = masks.mask_rows(kind, S, **kw)
+    rows = torch.tensor([0, 1, 63, 64, S // 2, S - 2, S - 1])
+    assert torch.equal(masks.mask_rows(kind, S, rows=rows, **kw), full[rows])
+
+
+# ------------------------------------------------------------------ pair counts
+@pytest.mark.parametrize("kind,S,kw", [
+    ("llm/scatter", 1000, dict(group_num=3)), ("llm/scatter", 2048, dict(group_num=8)),
+    ("llm/gather1", 1024, dict(group_num=8)), ("llm/gather1", 1000, dict(group_num=8)),
+    ("llm/window", 1000, dict(window=576)), ("llm/window", 3000, dict(window=1000)),
+    ("image/scatter", 4608, dict(width=64)), ("image/gather0", 4608, dict(width=64))])
+def test_pair_counts_equal_mask_sums(kind, S, kw):
+    assert pairs.pairs_per_head(kind, S, **kw) == int(masks.mask_rows(kind, S, **kw).sum())
+
+
+def test_pair_counts_headline():
+    assert pairs.pairs_per_head("llm/scatter", 32768, group_num=8) == 8 * (4096 * 4097 // 2) == 67125248
+    assert pairs.pairs_per_head("image/scatter", 16896, width=128) == 16896 * (512 + 2048)
+
+
+# ------------------------------------------------------------------ attention
+def _rand(B, S, H, Hkv, D, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, S, H, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, S, Hkv, D, generator=g).to(torch.bfloat16)
+    return q, k, v
+
+
+def test_attention_vs_float64_loops():
+    B, S, H, Hkv, D = 1, 24, 4, 2, 8
+    q, k, v = _rand(B, S, H, Hkv, D, 1)
+    q, k, v = q.float(), k.float(), v.float()
+    mask = masks.llm_scatter_mask(S, 3)
+    got = oracle.masked_attention(q, k, v, mask, softmax_scale=0.3)
+    for h in range(H):
+        kh = h // (H // Hkv)
+        for i in range(S):
+            js = [j for j in range(S) if mask[i, j]]
+            sc = [0.3 * sum(float(q[0, i, h, d]) * float(k[0, j, kh, d]) for d in range(D)) for j in js]
+            mx = max(sc)
+            w = [math.exp(s - mx) for s in sc]
+            z = sum(w)
+            for d in range(D):
+                want = sum(wi * float(v[0, j, kh, d]) for wi, j in zip(w, js)) / z
+                assert abs(float(got[0, i, h, d]) - want) < 1e-5
+
+
+@pytest.mark.parametrize("B,S,H,Hkv,kind,kw", [
+    (1, 1024, 4, 1, "llm/scatter", dict(group_num=8)),   # BASELINE config 1
+    (2, 300, 6, 2, "llm/window", dict(window=100)),
+    (1, 320, 3, 3, "image/gather0", dict(width=16, text_len=64))])
+def test_attention_vs_torch_sdpa(B, S, H, Hkv, kind, kw):
+    # same call shape as reference.py:78-83
+    q, k, v = _rand(B, S, H, Hkv, 128, 0)
+    mask = masks.mask_rows(kind, S, **kw)
+    got = oracle.masked_attention(q, k, v, mask)
+    qf, kf, vf = (x.float().transpose(1, 2) for x in (q, k, v))
+    ref = F.scaled_dot_product_attention(qf, kf, vf, attn_mask=mask, enable_gqa=H != Hkv)
+    ref = ref.transpose(1, 2).to(q.dtype)
+    assert got.dtype == q.dtype and got.shape == q.shape
+    assert (got.float() - ref.float()).abs().max().item() <= 2 ** -8  # one bf16 ulp at |x| < 1
+
+
+def test_attention_rows_subset_and_scale():
+    q, k, v = _rand(1, 200, 4, 2, 128, 3)
+    mask = masks.llm_scatter_mask(200, 2)
+    full = oracle.masked_attention(q, k, v, mask, softmax_scale=0.05)
+    rows = torch.tensor([0, 7, 64, 199])
+    sub = oracle.masked_attention_rows(q, k, v, mask[rows], rows, softmax_scale=0.05)
+    assert torch.equal(sub, full[:, rows])
+    assert not torch.equal(full, oracle.masked_attention(q, k, v, mask))

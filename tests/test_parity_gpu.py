@@ -1,0 +1,226 @@
+"""Parity of every kernel against the fp32 dense-mask oracle, through the Python API and the
+C ABI behind it.  Case matrix of the reference's tests/test_kernel.py:33-51 plus the BASELINE
+shapes, ragged / tiny / strided inputs and size-independent properties at full length.
+
+Tolerance: max-abs error <= 1.6e-2 on bf16 outputs (README.md:68-69 of the reference; its own
+test uses 2e-2 and reports ~1e-3 observed)."""
+import pytest
+import torch
+
+import oracle
+from intra_amd import intra_image_attn, intra_llm_attn
+
+pytestmark = pytest.mark.gpu
+ATOL = 1.6e-2
+DEV = "cuda"
+
+
+def make_qkv(B, S, H, Hkv, seed=0):
+    """i.i.d. N(0,1) drawn on the CPU from a fixed seed, rounded to bf16, then moved."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    q = torch.randn(B, S, H, 128, generator=g, dtype=torch.float32).to(torch.bfloat16)
+    k = torch.randn(B, S, Hkv, 128, generator=g, dtype=torch.float32).to(torch.bfloat16)
+    v = torch.randn(B, S, Hkv, 128, generator=g, dtype=torch.float32).to(torch.bfloat16)
+    return q.to(DEV), k.to(DEV), v.to(DEV)
+
+
+def check(out, q, k, v, kind, rows=None, scale=None, **kw):
+    S = q.shape[1]
+    assert out.shape == q.shape and out.dtype == torch.bfloat16
+    assert bool(torch.isfinite(out).all())
+    mask = oracle.mask_rows(kind, S, rows=rows, device=DEV, **kw)
+    ref = oracle.masked_attention_rows(q, k, v, mask, rows, softmax_scale=scale)
+    got = out if rows is None else out[:, rows]
+    err = (got.float() - ref.float()).abs().max().item()
+    assert err <= ATOL, f"{kind} {kw} S={S}: max|err|={err:.3e}"
+    return err
+
+
+HEADS = [(1, 32, 8), (2, 32, 32)]
+SEQS = [1000, 2048, 3000, 4096, 8192, 16384]
+
+
+@pytest.mark.parametrize("S", SEQS)
+@pytest.mark.parametrize("B,H,Hkv", HEADS)
+@pytest.mark.parametrize("G", [2, 3, 8])
+def test_llm_scatter(S, B, H, Hkv, G):
+    q, k, v = make_qkv(B, S, H, Hkv)
+    with torch.no_grad():
+        out = intra_llm_attn(q, k, v, "scatter", group_num=G)
+    check(out, q, k, v, "llm/scatter", group_num=G)
+
+
+@pytest.mark.parametrize("S", [s for s in SEQS if s % 64 == 0])
+@pytest.mark.parametrize("B,H,Hkv", HEADS)
+def test_llm_gather1(S, B, H, Hkv):
+    q, k, v = make_qkv(B, S, H, Hkv)
+    with torch.no_grad():
+        out = intra_llm_attn(q, k, v, "gather1", group_num=8)
+    check(out, q, k, v, "llm/gather1", group_num=8)
+
+
+@pytest.mark.parametrize("S", SEQS)
+@pytest.mark.parametrize("B,H,Hkv", HEADS)
+@pytest.mark.parametrize("W", [576, 1000])
+def test_llm_window(S, B, H, Hkv, W):
+    q, k, v = make_qkv(B, S, H, Hkv)
+    with torch.no_grad():
+        out = intra_llm_attn(q, k, v, "window", window=W)
+    check(out, q, k, v, "llm/window", window=W)
+
+
+@pytest.mark.parametrize("width,H", [(64, 24), (128, 8)])
+@pytest.mark.parametrize("B", [1, 2])
+@pytest.mark.parametrize("pattern", ["scatter", "gather0"])
+def test_image(width, H, B, pattern):
+    S = 512 + width * width
+    q, k, v = make_qkv(B, S, H, H)
+    with torch.no_grad():
+        out = intra_image_attn(q, k, v, pattern, width)
+    check(out, q, k, v, f"image/{pattern}", width=width)
+
+
+def test_baseline_config1_shape():
+    # S=1024, 4 query heads / 1 kv head, Scatter G=8
+    q, k, v = make_qkv(1, 1024, 4, 1)
+    with torch.no_grad():
+        out = intra_llm_attn(q, k, v, "scatter", group_num=8)
+    check(out, q, k, v, "llm/scatter", group_num=8)
+
+
+@pytest.mark.parametrize("S,pattern,kw", [
+    (1, "scatter", dict(group_num=8)), (5, "scatter", dict(group_num=8)),
+    (63, "scatter", dict(group_num=1)), (65, "scatter", dict(group_num=1)),
+    (257, "scatter", dict(group_num=2)), (777, "scatter", dict(group_num=16)),
+    (64, "gather1", dict(group_num=8)), (128, "gather1", dict(group_num=8)),
+    (1, "window", dict(window=576)), (100, "window", dict(window=64)),
+    (1000, "window", dict(window=65)), (300, "window", dict(window=5000)),
+    (1000, "window", dict(window=130))])
+@pytest.mark.parametrize("H,Hkv", [(4, 1), (2, 1), (3, 3), (8, 1)])
+def test_llm_ragged_and_tiny(S, pattern, kw, H, Hkv):
+    q, k, v = make_qkv(2, S, H, Hkv, seed=S)
+    with torch.no_grad():
+        out = intra_llm_attn(q, k, v, pattern, **kw)
+    check(out, q, k, v, f"llm/{pattern}", **kw)
+
+
+@pytest.mark.parametrize("H,Hkv", [(8, 2), (4, 2)])
+@pytest.mark.parametrize("pattern", ["scatter", "gather0"])
+def test_image_gqa(H, Hkv, pattern):
+    q, k, v = make_qkv(1, 4608, H, Hkv, seed=5)
+    with torch.no_grad():
+        out = intra_image_attn(q, k, v, pattern, 64)
+    check(out, q, k, v, f"image/{pattern}", width=64)
+
+
+def test_strided_views_and_scale():
+    # (B, H, S, D) storage viewed as (B, S, H, D): head stride S*128, as a FLUX-style caller passes
+    B, S, H, Hkv = 2, 1000, 8, 2
+    q, k, v = make_qkv(B, S, H, Hkv, seed=11)
+    qt = q.transpose(1, 2).contiguous().transpose(1, 2)
+    kt = k.transpose(1, 2).contiguous().transpose(1, 2)
+    vt = v.transpose(1, 2).contiguous().transpose(1, 2)
+    assert qt.stride(2) == S * 128
+    with torch.no_grad():
+        out = intra_llm_attn(qt, kt, vt, "scatter", group_num=3, softmax_scale=0.05)
+        base = intra_llm_attn(q, k, v, "scatter", group_num=3, softmax_scale=0.05)
+    assert out.stride() == qt.stride()
+    assert torch.equal(out, base)
+    check(out, q, k, v, "llm/scatter", scale=0.05, group_num=3)
+    # sliced out of a fused qkv buffer: batch/row strides larger than the tensor
+    fused = torch.zeros(B, S, H + 2 * Hkv, 128, dtype=torch.bfloat16, device=DEV)
+    fused[:, :, :H], fused[:, :, H:H + Hkv], fused[:, :, H + Hkv:] = q, k, v
+    with torch.no_grad():
+        out2 = intra_llm_attn(fused[:, :, :H], fused[:, :, H:H + Hkv], fused[:, :, H + Hkv:], "scatter",
+                              group_num=3, softmax_scale=0.05)
+    assert torch.equal(out2, base)
+
+
+@pytest.mark.parametrize("scale", [-0.07, 0.0, 0.3])
+def test_unusual_scales(scale):
+    q, k, v = make_qkv(1, 512, 4, 4, seed=2)
+    with torch.no_grad():
+        out = intra_llm_attn(q, k, v, "window", window=128, softmax_scale=scale)
+    check(out, q, k, v, "llm/window", scale=scale, window=128)
+
+
+def test_deterministic_and_async_on_side_stream():
+    q, k, v = make_qkv(1, 4096, 32, 8, seed=4)
+    with torch.no_grad():
+        a = intra_llm_attn(q, k, v, "scatter", group_num=8)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            b = intra_llm_attn(q, k, v, "scatter", group_num=8)
+        side.synchronize()
+    assert torch.equal(a, b)
+
+
+def _row_subset(S, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    rows = torch.randperm(S, generator=g)[:n]
+    edge = torch.tensor([0, 1, 63, 64, S - 65, S - 64, S - 1])
+    return torch.unique(torch.cat([rows, edge])).to(DEV)
+
+
+@pytest.mark.parametrize("S", [32768, 65536])
+@pytest.mark.parametrize("pattern,kw", [("scatter", dict(group_num=8)), ("scatter", dict(group_num=2)),
+                                        ("gather1", dict(group_num=8)), ("window", dict(window=576))])
+def test_llm_full_length_row_subset(S, pattern, kw):
+    q, k, v = make_qkv(1, S, 32, 8, seed=1)
+    with torch.no_grad():
+        out = intra_llm_attn(q, k, v, pattern, **kw)
+    check(out, q, k, v, f"llm/{pattern}", rows=_row_subset(S, 1024, S), **kw)
+
+
+@pytest.mark.parametrize("pattern", ["scatter", "gather0"])
+def test_image_2048_row_subset(pattern):
+    S = 512 + 128 * 128
+    q, k, v = make_qkv(1, S, 24, 24, seed=3)
+    with torch.no_grad():
+        out = intra_image_attn(q, k, v, pattern, 128)
+    rows = torch.unique(torch.cat([_row_subset(S, 1024, 7), torch.arange(0, 512, 5, device=DEV),
+                                   torch.tensor([512, 512 + 127, S - 128], device=DEV)]))
+    check(out, q, k, v, f"image/{pattern}", rows=rows, width=128)
+
+
+def test_scatter_groups_are_independent_at_full_length():
+    """Size-independent property: Scatter over S tokens equals G separate dense causal problems,
+    so running the kernel on the de-interleaved tokens of one group with G=1 must reproduce that
+    group's rows bit for bit."""
+    S, G = 32768, 8
+    q, k, v = make_qkv(1, S, 32, 8, seed=9)
+    with torch.no_grad():
+        full = intra_llm_attn(q, k, v, "scatter", group_num=G)
+        for g in (0, 5):
+            sub = intra_llm_attn(q[:, g::G], k[:, g::G], v[:, g::G], "scatter", group_num=1)
+            assert torch.equal(sub, full[:, g::G])
+
+
+def test_api_errors_on_gpu_tensors():
+    q, k, v = make_qkv(1, 1000, 4, 4)
+    with pytest.raises(ValueError, match="gather1 needs group_num=8"):
+        intra_llm_attn(q, k, v, "gather1", group_num=8)
+    with pytest.raises(ValueError, match="gather1 needs group_num=8"):
+        intra_llm_attn(q[:, :960], k[:, :960], v[:, :960], "gather1", group_num=4)
+    with pytest.raises(KeyError):
+        intra_llm_attn(q, k, v, "gather0")
+    with pytest.raises(ValueError, match="width 64 and 128"):
+        intra_image_attn(q, k, v, "scatter", 32)
+    with pytest.raises(ValueError, match="expected 512 text"):
+        intra_image_attn(q, k, v, "scatter", 64)
+    with pytest.raises(RuntimeError, match="window must be >= 64"):
+        intra_llm_attn(q, k, v, "window", window=32)
+    qg = q.clone().requires_grad_(True)
+    with pytest.raises(RuntimeError, match="forward-only"):
+        intra_llm_attn(qg, k, v)
+    with torch.no_grad():
+        intra_llm_attn(qg, k, v)
+
+
+def test_oracle_on_gpu_equals_oracle_on_cpu():
+    q, k, v = make_qkv(1, 1024, 4, 1)
+    mask = oracle.llm_scatter_mask(1024, 8)
+    a = oracle.masked_attention(q.cpu(), k.cpu(), v.cpu(), mask)
+    b = oracle.masked_attention(q, k, v, mask.to(DEV)).cpu()
+    assert (a.float() - b.float()).abs().max().item() <= 2 ** -8
