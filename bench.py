@@ -1,0 +1,127 @@
+"""Headline benchmark: LLM causal Scatter G=8 at S=32768 (B=1, 32 query / 8 kv heads, d=128,
+bf16) on one MI355X.  A step is one call of intra_llm_attn on inputs already resident in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--seqlen S] [--no-cpu]
+
+Prints ONE JSON line.  `value` is effective TFLOP/s (flops of unmasked query-key pairs only,
+4*128 per pair and head) over the wall-clock of the K timed steps; `roofline` is the same
+algorithmic work over the kernel's own average duration (HIP events on the launch stream);
+`cpu_baseline` is the fp32 dense-mask oracle on the host cores for a bounded sample of query rows
+of the same problem.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU; AMD publishes it as 2.5 PFLOP/s dense
+# HBM bytes per launch at S=32768 measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/); None until measured for the current kernel.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--seqlen", type=int, default=32768)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the kernels are single-GPU and this build launches nothing "
+                 "across GPUs; run with --gpus 1")
+
+    import torch
+
+    import oracle
+    from intra_amd import _lib, intra_llm_attn
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    assert os.path.exists(_lib.LIB_PATH), "libintra_hip.so is not built"
+    dev = torch.device("cuda:0")
+    B, S, H, Hkv, G = 1, args.seqlen, 32, 8, 8
+    g = torch.Generator(device="cpu").manual_seed(0)
+    mk = lambda h: torch.randn(B, S, h, 128, generator=g, dtype=torch.float32).to(torch.bfloat16)
+    q_cpu, k_cpu, v_cpu = mk(H), mk(Hkv), mk(Hkv)
+    q, k, v = q_cpu.to(dev), k_cpu.to(dev), v_cpu.to(dev)
+    pairs = oracle.pairs_per_head("llm/scatter", S, group_num=G)
+    flop = 4.0 * 128 * pairs * H * B
+
+    step = lambda: intra_llm_attn(q, k, v, "scatter", group_num=G)
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            out = step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = step()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+        # per-launch kernel duration: HIP events on the stream the kernel is launched on
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+               for _ in range(args.steps)]
+        for a, b in evs:
+            a.record()
+            step()
+            b.record()
+        torch.cuda.synchronize()
+        kern_ms = sorted(a.elapsed_time(b) for a, b in evs)
+    kern_avg = sum(kern_ms) / len(kern_ms)
+
+    # parity spot check on a row subset so that a wrong kernel cannot post a number
+    rows = torch.unique(torch.cat([torch.randperm(S, generator=g)[:256], torch.tensor([0, S - 1])])).to(dev)
+    ref = oracle.masked_attention_rows(q, k, v, oracle.llm_scatter_mask(S, G, dev, rows), rows)
+    err = (out[:, rows].float() - ref.float()).abs().max().item()
+    assert err <= 1.6e-2, f"parity failed in bench: {err}"
+
+    tflops = flop / (wall_ms * 1e-3) / 1e12
+    achieved = flop / (kern_avg * 1e-3) / 1e12
+    res = {
+        "metric": "Scatter G=8 32K ms/call + effective TFLOP/s (% bf16 MFMA peak), 1 MI355X",
+        "value": round(tflops, 2), "unit": "effective TFLOP/s (unmasked pairs only)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic: i.i.d. N(0,1) from CPU seed 0, rounded to bf16",
+        "config": {"workload": f"LLM causal Scatter G={G}, B={B}, S={S}, {H} query / {Hkv} kv heads, d=128",
+                   "pairs_per_head": pairs, "tflop_per_call": round(flop / 1e12, 6)},
+        "ms_per_call": round(wall_ms, 4), "pct_of_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
+        "kernel_ms": {"avg": round(kern_avg, 4), "median": round(kern_ms[len(kern_ms) // 2], 4),
+                      "min": round(kern_ms[0], 4), "p90": round(kern_ms[int(0.9 * (len(kern_ms) - 1))], 4)},
+        "parity_max_abs_err": err,
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(S)},
+        "device": torch.cuda.get_device_name(0),
+        "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
+    }
+
+    if not args.no_cpu:
+        # Bounded sample of the same problem: evenly spaced query rows of all heads against all
+        # keys through the dense-mask fp32 path, on the host cores.
+        n_rows = 1024 if S >= 8192 else S
+        rows_c = torch.arange(0, S, S // n_rows)[:n_rows]
+        mask_c = oracle.llm_scatter_mask(S, G, rows=rows_c)
+        cores = torch.get_num_threads()
+        oracle.masked_attention_rows(q_cpu, k_cpu, v_cpu, mask_c[:64], rows_c[:64], chunk=64)  # warm-up
+        t0 = time.perf_counter()
+        oracle.masked_attention_rows(q_cpu, k_cpu, v_cpu, mask_c, rows_c, chunk=128)
+        dt = time.perf_counter() - t0
+        eff = 4.0 * 128 * int(mask_c.sum()) * H * B
+        res["cpu_baseline"] = {
+            "value": round(eff / dt / 1e12, 6), "unit": "effective TFLOP/s (unmasked pairs only)",
+            "cores": cores, "kind": "port",
+            "sample": f"{n_rows} evenly spaced query rows x {H} heads of the same S={S} problem, dense-mask fp32 "
+                      f"oracle, {dt:.2f} s; dense work {4.0 * 128 * n_rows * S * H / dt / 1e12:.4f} TFLOP/s",
+        }
+    print(json.dumps(res), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,141 @@
+"""Per-pattern latency table of the INTRA kernels on MI355X.
+
+Same protocol and CLI as the reference's benchmarks/bench_kernel.py:23-34,91-111 (median of
+--iters event-timed calls after --warmup calls; `llm` and `image` modes), with the rows extended
+by effective TFLOP/s (unmasked pairs only) and the fraction of the bf16 dense MFMA peak.
+
+    python -m intra_amd.bench_kernel llm   --seqlens 4096,8192,16384,32768,65536
+    python -m intra_amd.bench_kernel image
+"""
+import argparse
+import json
+
+import torch
+import torch.nn.functional as F
+
+from intra_amd import _lib, intra_image_attn, intra_llm_attn
+from intra_amd.interface import TEXT_LEN
+
+PEAK_BF16_TFLOPS = 2516.6
+
+
+def median_ms(fn, warmup, iters):
+    for _ in range(warmup):
+        fn()
+    times = []
+    for _ in range(iters):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        end.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(end))
+    return sorted(times)[len(times) // 2]
+
+
+def pairs(domain, pattern, B, S, H, Hkv, a0, a1):
+    import ctypes
+    plan = _lib.IntraPlan()
+    rc = _lib.load().intra_plan(domain, pattern, B, S, H, Hkv, a0, a1, ctypes.byref(plan))
+    assert rc == 0, _lib.last_error()
+    return plan.pairs_per_head
+
+
+def dense_sdpa(q, k, v, causal):
+    q, k, v = (x.transpose(1, 2) for x in (q, k, v))
+    return F.scaled_dot_product_attention(q, k, v, is_causal=causal, enable_gqa=q.shape[1] != k.shape[1])
+
+
+def qkv(B, S, H, Hkv, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    mk = lambda h: torch.randn(B, S, h, 128, generator=g).to(torch.bfloat16).cuda()
+    return mk(H), mk(Hkv), mk(Hkv)
+
+
+def entry(ms, npairs, B, H):
+    tf = 4 * 128 * npairs * H * B / (ms * 1e-3) / 1e12
+    return {"ms": round(ms, 4), "tflops_eff": round(tf, 1), "pct_peak": round(100 * tf / PEAK_BF16_TFLOPS, 1)}
+
+
+@torch.no_grad()
+def bench_llm(args):
+    rows = []
+    B, H, Hkv = args.batch, args.heads, args.kv_heads
+    for S in args.seqlens:
+        q, k, v = qkv(B, S, H, Hkv)
+        r = {"seqlen": S}
+        if args.dense:
+            ms = median_ms(lambda: dense_sdpa(q, k, v, True), args.warmup, args.iters)
+            r["dense"] = entry(ms, S * (S + 1) // 2, B, H)
+        for G in args.groups:
+            ms = median_ms(lambda: intra_llm_attn(q, k, v, "scatter", group_num=G), args.warmup, args.iters)
+            r[f"scatter_g{G}"] = entry(ms, pairs(0, 0, B, S, H, Hkv, G, 576), B, H)
+        if S % 64 == 0:
+            ms = median_ms(lambda: intra_llm_attn(q, k, v, "gather1", group_num=8), args.warmup, args.iters)
+            r["gather1_g8"] = entry(ms, pairs(0, 1, B, S, H, Hkv, 8, 576), B, H)
+        ms = median_ms(lambda: intra_llm_attn(q, k, v, "window", window=576), args.warmup, args.iters)
+        r["window576"] = entry(ms, pairs(0, 4, B, S, H, Hkv, 8, 576), B, H)
+        if "scatter_g2" in r:
+            # the reference's arithmetic for the 32-layer g2s4 schedule (bench_kernel.py:66-68) ...
+            r["g2s4_32layer_ms"] = round(4 * r["scatter_g2"]["ms"] + 28 * r["window576"]["ms"], 3)
+            # ... and the same stack actually run back to back with fresh inputs per layer
+            layers = [qkv(B, S, H, Hkv, seed=i) for i in range(4)]
+
+            def stack():
+                for i in range(32):
+                    ql, kl, vl = layers[i % 4]
+                    if i % 8 == 0:
+                        intra_llm_attn(ql, kl, vl, "scatter", group_num=2)
+                    else:
+                        intra_llm_attn(ql, kl, vl, "window", window=576)
+            r["g2s4_32layer_run_ms"] = round(median_ms(stack, 2, max(3, args.iters // 10)), 3)
+        rows.append(r)
+        print(json.dumps(r), flush=True)
+    return rows
+
+
+@torch.no_grad()
+def bench_image(args):
+    rows = []
+    B, H = args.batch, args.image_heads
+    for width in (64, 128):
+        S = TEXT_LEN + width * width
+        q, k, v = qkv(B, S, H, H)
+        r = {"width": width, "seqlen": S}
+        if args.dense:
+            r["dense"] = entry(median_ms(lambda: dense_sdpa(q, k, v, False), args.warmup, args.iters), S * S, B, H)
+        for pattern, pid in (("scatter", 0), ("gather0", 4)):
+            ms = median_ms(lambda: intra_image_attn(q, k, v, pattern, width), args.warmup, args.iters)
+            r[pattern] = entry(ms, pairs(1, pid, B, S, H, H, width, TEXT_LEN), B, H)
+        r["interleaved_mean_ms"] = round((r["scatter"]["ms"] + r["gather0"]["ms"]) / 2, 4)
+        rows.append(r)
+        print(json.dumps(r), flush=True)
+    return rows
+
+
+def main():
+    p = argparse.ArgumentParser()
+    p.add_argument("mode", choices=["llm", "image"])
+    p.add_argument("--seqlens", default="4096,8192,16384,32768,65536")
+    p.add_argument("--groups", default="2,8")
+    p.add_argument("--batch", type=int, default=1)
+    p.add_argument("--heads", type=int, default=32)
+    p.add_argument("--kv-heads", type=int, default=8)
+    p.add_argument("--image-heads", type=int, default=24)
+    p.add_argument("--warmup", type=int, default=10)
+    p.add_argument("--iters", type=int, default=50)
+    p.add_argument("--dense", action="store_true", help="also time torch SDPA on the dense problem")
+    p.add_argument("--out", help="optional JSON output path")
+    args = p.parse_args()
+    args.seqlens = [int(x) for x in args.seqlens.split(",")]
+    args.groups = [int(x) for x in args.groups.split(",")]
+    print(f"device: {torch.cuda.get_device_name()}  torch {torch.__version__}  peak {PEAK_BF16_TFLOPS} TFLOP/s")
+    rows = bench_llm(args) if args.mode == "llm" else bench_image(args)
+    if args.out:
+        json.dump({"device": torch.cuda.get_device_name(), "torch": torch.__version__,
+                   "args": {k: v for k, v in vars(args).items() if k != "out"}, "rows": rows},
+                  open(args.out, "w"), indent=1)
+
+
+if __name__ == "__main__":
+    main()
