@@ -32,6 +32,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--seqlen", type=int, default=32768)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also run three plain 1 GiB device copies, the known-size kernel that scales "
+                         "FETCH_SIZE / WRITE_SIZE readings of a counter run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the kernels are single-GPU and this build launches nothing "
@@ -52,6 +55,14 @@ def main():
     q, k, v = q_cpu.to(dev), k_cpu.to(dev), v_cpu.to(dev)
     pairs = oracle.pairs_per_head("llm/scatter", S, group_num=G)
     flop = 4.0 * 128 * pairs * H * B
+
+    if args.copy_calib:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     step = lambda: intra_llm_attn(q, k, v, "scatter", group_num=G)
     with torch.no_grad():

@@ -3,7 +3,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libintra_hip.so")
+# INTRA_HIP_LIB overrides the in-tree build (e.g. to try another build of the same ABI)
+LIB_PATH = os.environ.get("INTRA_HIP_LIB") or os.path.join(_HERE, "libintra_hip.so")
 
 INTRA_OK, INTRA_ERR_INVALID, INTRA_ERR_UNSUPPORTED, INTRA_ERR_HIP = 0, 1, 2, 3
 

@@ -100,7 +100,7 @@ void fill_plan(const Request& r, int hp, int nw, IntraPlan* plan) {
   const int64_t n_pairs = (int64_t)r.B * r.Hkv * plan->n_sets;
   const int64_t grid = 8 * ((n_pairs + 7) / 8) * hgroups * plan->n_mblocks;
   plan->grid = grid > 0x7fffffff ? -1 : (int)grid;
-  plan->lds_bytes = 2 * intra::BUF_BYTES;
+  plan->lds_bytes = intra::LDS_BYTES;
   int64_t pairs = 0;
   for (int set = 0; set < plan->n_sets; ++set) {
     MAP map(r.geom, set);
@@ -241,7 +241,17 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   float c = fabsf(scale) * 1.4426950408889634f;
   if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights without 0 * inf
   p.scale_log2 = c;
+  p.rescale_gap = 8.0f / c;
   p.negate_q = scale < 0.f;
+  {
+    // 32-bit gather offsets: position < 2^24, row stride in bytes < 2^24, last row below 4 GiB
+    const int64_t krb = ks[1] * 2, vrb = vs[1] * 2;
+    const int64_t lim = (int64_t)1 << 32;
+    p.small_offsets = S < (1 << 24) && krb < (1 << 24) && vrb < (1 << 24) &&
+                      (int64_t)S * krb + 256 < lim && (int64_t)S * vrb + 256 < lim;
+    p.k_rs_bytes = (uint32_t)(krb & 0xffffffff);
+    p.v_rs_bytes = (uint32_t)(vrb & 0xffffffff);
+  }
   p.n_sets = plan.n_sets;
   p.n_mblocks = plan.n_mblocks;
   p.hgroups = p.ratio / hp;
