@@ -75,7 +75,8 @@ typedef struct IntraPlan {
   int pos_per_block;   /* in-set queries per workgroup */
   int n_sets;          /* sets per (batch, kv head) */
   int n_mblocks;       /* row blocks of the largest set */
-  int grid;            /* workgroups launched */
+  int work_items;      /* row blocks to process (a multiple of 8: padded per XCD) */
+  int grid;            /* upper bound of workgroups launched: min(work_items, CUs of the device) */
   int lds_bytes;       /* LDS per workgroup */
   int64_t pairs_per_head; /* unmasked (query, key) pairs per query head and batch */
 } IntraPlan;

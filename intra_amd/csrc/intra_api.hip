@@ -98,8 +98,9 @@ void fill_plan(const Request& r, int hp, int nw, IntraPlan* plan) {
   plan->n_mblocks = (MAP::max_nq(r.geom) + pos - 1) / pos;
   const int hgroups = (r.H / r.Hkv) / hp;
   const int64_t n_pairs = (int64_t)r.B * r.Hkv * plan->n_sets;
-  const int64_t grid = 8 * ((n_pairs + 7) / 8) * hgroups * plan->n_mblocks;
-  plan->grid = grid > 0x7fffffff ? -1 : (int)grid;
+  const int64_t items = 8 * ((n_pairs + 7) / 8) * hgroups * plan->n_mblocks;
+  plan->work_items = items > 0x7fffffff ? -1 : (int)items;
+  plan->grid = plan->work_items;  // upper bound; a launch uses min(work_items, 8 * (CUs / 8))
   plan->lds_bytes = intra::LDS_BYTES;
   int64_t pairs = 0;
   for (int set = 0; set < plan->n_sets; ++set) {
@@ -173,6 +174,21 @@ void model_walk(const IntraGeom& ge, int hp, int nw, uint8_t* count) {
   }
 }
 
+// One persistent workgroup per CU (LDS allows no more), in multiples of the 8 XCDs.
+int launch_grid(int work_items) {
+  static int cus[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
+  if (cus[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return -1;
+    cus[dev] = n;
+  }
+  int g = (cus[dev] / 8) * 8;
+  if (g < 8) g = 8;
+  return work_items < g ? work_items : g;
+}
+
 template <class MAP, int HP, int NW>
 int launch(const intra::KParams& p, int grid, hipStream_t stream) {
   hipLaunchKernelGGL((intra::intra_fwd_kernel<MAP, HP, NW>), dim3(grid), dim3(NW * 64), 0, stream, p);
@@ -225,7 +241,9 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   pick_shape(r.kind, H / Hkv, &hp, &nw);
   IntraPlan plan;
   plan_for(r, hp, nw, &plan);
-  if (plan.grid <= 0) return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 workgroups");
+  if (plan.work_items <= 0) return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 work items");
+  const int grid = launch_grid(plan.work_items);
+  if (grid <= 0) return fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
 
   intra::KParams p;
   p.q = static_cast<const uint16_t*>(q);
@@ -238,37 +256,31 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.o_bs = os[0]; p.o_rs = os[1]; p.o_hs = os[2];
   p.B = B; p.H = H; p.Hkv = Hkv; p.ratio = H / Hkv;
   p.geom = r.geom;
-  float c = fabsf(scale) * 1.4426950408889634f;
-  if (c < 1e-30f) c = 1e-30f;  // scale 0: uniform weights without 0 * inf
-  p.scale_log2 = c;
-  p.rescale_gap = 8.0f / c;
+  p.scale_log2 = fabsf(scale) * 1.4426950408889634f;
+  if (p.scale_log2 < 1e-30f) p.scale_log2 = 1e-30f;  // scale 0: uniform weights without 0 * inf on masked scores
   p.negate_q = scale < 0.f;
-  {
-    // 32-bit gather offsets: position < 2^24, row stride in bytes < 2^24, last row below 4 GiB
-    const int64_t krb = ks[1] * 2, vrb = vs[1] * 2;
-    const int64_t lim = (int64_t)1 << 32;
-    p.small_offsets = S < (1 << 24) && krb < (1 << 24) && vrb < (1 << 24) &&
-                      (int64_t)S * krb + 256 < lim && (int64_t)S * vrb + 256 < lim;
-    p.k_rs_bytes = (uint32_t)(krb & 0xffffffff);
-    p.v_rs_bytes = (uint32_t)(vrb & 0xffffffff);
-  }
+  if (ks[1] >= ((int64_t)1 << 31) || vs[1] >= ((int64_t)1 << 31))
+    return fail(INTRA_ERR_UNSUPPORTED, "k / v token stride must stay below 2^31 elements");
+  p.k_rs_bytes = (uint32_t)(ks[1] * 2);
+  p.v_rs_bytes = (uint32_t)(vs[1] * 2);
   p.n_sets = plan.n_sets;
   p.n_mblocks = plan.n_mblocks;
   p.hgroups = p.ratio / hp;
   p.n_pairs = B * Hkv * plan.n_sets;
   p.items_per_pair = p.hgroups * plan.n_mblocks;
+  p.n_slots = plan.work_items / 8;
 
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (r.kind) {
-    case KIND_LLM_SCATTER: return launch_hp8<MapLlmScatter>(p, hp, plan.grid, st);
-    case KIND_LLM_GATHER1: return launch_hp8<MapLlmGather1>(p, hp, plan.grid, st);
-    case KIND_LLM_WINDOW: return launch_hp8<MapLlmWindow>(p, hp, plan.grid, st);
-    case KIND_IMG_SCATTER: return launch_hp8<MapImgScatter>(p, hp, plan.grid, st);
+    case KIND_LLM_SCATTER: return launch_hp8<MapLlmScatter>(p, hp, grid, st);
+    case KIND_LLM_GATHER1: return launch_hp8<MapLlmGather1>(p, hp, grid, st);
+    case KIND_LLM_WINDOW: return launch_hp8<MapLlmWindow>(p, hp, grid, st);
+    case KIND_IMG_SCATTER: return launch_hp8<MapImgScatter>(p, hp, grid, st);
     default:
       switch (hp) {
-        case 4: return launch<MapImgGather0, 4, 8>(p, plan.grid, st);
-        case 2: return launch<MapImgGather0, 2, 4>(p, plan.grid, st);
-        default: return launch<MapImgGather0, 1, 2>(p, plan.grid, st);
+        case 4: return launch<MapImgGather0, 4, 8>(p, grid, st);
+        case 2: return launch<MapImgGather0, 2, 4>(p, grid, st);
+        default: return launch<MapImgGather0, 1, 2>(p, grid, st);
       }
   }
 }

@@ -55,25 +55,50 @@ struct KParams {
   int64_t o_bs, o_rs, o_hs;
   int B, H, Hkv, ratio;
   IntraGeom geom;
-  float scale_log2;    // |softmax_scale| * log2(e), > 0
-  float rescale_gap;   // raw-score gap that forces a new reference maximum: 8 / scale_log2
+  float scale_log2;    // |softmax_scale| * log2(e)
   int negate_q;        // softmax_scale < 0: flip the sign of Q instead
-  int small_offsets;   // K/V row offsets fit 32 bits and the factors 24 bits
-  uint32_t k_rs_bytes, v_rs_bytes;
+  uint32_t k_rs_bytes, v_rs_bytes;  // token strides of k and v in bytes (< 4 GiB, checked on the host)
   int n_sets;          // sets per (batch, kv head)
   int n_mblocks;       // row blocks of the largest set
   int hgroups;         // ratio / HP
   int n_pairs;         // B * Hkv * n_sets
   int items_per_pair;  // hgroups * n_mblocks
+  int n_slots;         // work items per XCD: ceil(n_pairs / 8) * items_per_pair
 };
 
-constexpr int BN = 64;            // keys per tile (one barrier per tile)
-constexpr int KSTRIDE = 272;      // bytes per K row in LDS: 16 consecutive rows hit 16 distinct 16-byte slots
-constexpr int VSTRIDE = 320;      // bytes per V row in LDS: 4 consecutive rows cover 4 distinct 64-byte spans
-constexpr int KTILE = BN * KSTRIDE;
-constexpr int VTILE = BN * VSTRIDE;
-constexpr int VBASE = 3 * KTILE;  // K[3] then V[2]
-constexpr int LDS_BYTES = 3 * KTILE + 2 * VTILE;
+constexpr int BN = 64;             // keys per tile (one barrier per tile)
+// LDS tile layout.  A tile is 16 groups of 4 rows; a group is 1024 contiguous bytes (what one
+// 16-bytes-per-lane direct-to-LDS load instruction writes) followed by 16 bytes of padding.
+// Inside a group, the 16-byte chunk c of row i (0..3) sits at chunk slot c ^ (4 * i).  With
+// that, 16 consecutive rows read at one chunk (the K operand pattern) and the 4 rows x 64 bytes
+// of a transposing V read both touch 16 distinct 16-byte bank groups.
+constexpr int GROUP_STRIDE = 1024 + 16;
+constexpr int TILE_BYTES = (BN / 4) * GROUP_STRIDE;
+constexpr int KTILE = TILE_BYTES;
+constexpr int VTILE = TILE_BYTES;
+constexpr int NKBUF = 4, NVBUF = 3;   // K tiles i-1 (being overwritten) .. i+2, V tiles i-1 .. i+1
+constexpr int VBASE = NKBUF * KTILE;  // K ring then V ring
+constexpr int LDS_BYTES = NKBUF * KTILE + NVBUF * VTILE;
+constexpr int BLOCK32 = 8 * GROUP_STRIDE;  // 32 rows
+
+// 64 lanes x 16 bytes from per-lane global addresses to 1024 consecutive LDS bytes at lds_addr
+// (wave-uniform).  Issued as inline assembly so that the compiler does not put a full vmcnt(0)
+// wait in front of every later LDS read; completion is tracked by hand with vmcnt (see the main
+// loop), and the "memory" clobber keeps LDS accesses from moving across it at compile time.
+__device__ __forceinline__ void dma_group(const void* gsrc, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gsrc), "s"(lds_addr) : "memory");
+}
+
+// Workgroup barrier that leaves the `pending` most recent direct-to-LDS loads of this wavefront
+// in flight: waits for all its LDS reads (so buffers it was reading may be overwritten) and for
+// all but `pending` of its loads (so older tiles are complete), then s_barrier.
+template <int PENDING>
+__device__ __forceinline__ void tile_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((PENDING & 15) | ((PENDING >> 4) << 14) | (7 << 4) | (0 << 8));
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
 
 __device__ __forceinline__ float lane_xor32_max(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -91,20 +116,33 @@ template <class MAP, int HP, int NW>
 __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   constexpr int NT = NW * 64;
   constexpr int POS = NW * 32 / HP;          // in-set queries per row block
-  constexpr int LD_PASSES = (BN * 16) / NT;  // 16-byte chunks per thread per tile (K or V)
-  static_assert((BN * 16) % NT == 0, "tile must split evenly over the threads");
+  static_assert(BN % NW == 0, "tile rows must split evenly over the wavefronts");
 
   __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
 
-  // ---------------------------------------------------------------- which work item is this?
-  // Workgroups are handed to the 8 XCDs round-robin by id.  All row blocks of one (batch, kv head,
-  // set) "pair" go to one XCD, one pair after the other, longest row block first, so that the
-  // pair's K/V stays in that XCD's L2 while its row blocks run.
-  const int wg = blockIdx.x;
-  const int xcd = wg & 7;
-  const int slot = wg >> 3;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h32 = lane >> 5;  // which half of the wavefront
+  const int l32 = lane & 31;
+
+  // ---------------------------------------------------------------- persistent loop over work items
+  // The grid holds about one workgroup per CU and every workgroup walks through several work items
+  // (row blocks), which saves the dispatch gap between consecutive workgroups on a CU.
+  // Workgroups are handed to the 8 XCDs round-robin by id, so workgroup id % 8 names the XCD.  All
+  // row blocks of one (batch, kv head, set) "pair" go to one XCD, one pair after the other, longest
+  // row block first, so that the pair's K/V stays in that XCD's L2 while its row blocks run.  Inside
+  // an XCD the slots are dealt to its workgroups in boustrophedon order (0..w-1, w-1..0, ...), which
+  // balances the triangular causal workloads.
+  const int xcd = blockIdx.x & 7;
+  const int wgs_per_xcd = gridDim.x >> 3;
+  const int wg_in_xcd = blockIdx.x >> 3;
+  for (int round = 0;; ++round) {
+  const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
+  if (slot >= p.n_slots) break;
+  if (round > 0) tile_barrier<0>();  // everybody is done with the LDS tiles of the previous item
   const int pair = (slot / p.items_per_pair) * 8 + xcd;
-  if (pair >= p.n_pairs) return;
+  if (pair >= p.n_pairs) continue;
   const int rem = slot % p.items_per_pair;
   const int mblk = p.n_mblocks - 1 - rem / p.hgroups;
   const int hg = rem % p.hgroups;
@@ -118,17 +156,11 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   const int nq = map.nq();
   const int nk = map.nk();
   const int t0 = mblk * POS;
-  if (t0 >= nq) return;
+  if (t0 >= nq) continue;
   const int t1 = im_min(t0 + POS, nq) - 1;
   const int kt_lo = map.klo(t0);
   const int kt_hi = im_min(map.khi(t1), nk - 1);
   const int ntiles = (kt_hi - kt_lo + BN) / BN;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int h32 = lane >> 5;  // which half of the wavefront
-  const int l32 = lane & 31;
 
   // ---------------------------------------------------------------- this wavefront's queries
   const int hw = wave % HP;
@@ -156,73 +188,56 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 
   // Q^T fragments: lane holds query l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
   bf16x8 qf[8];
-  {
-    const uint16_t* qrow = p.q + batch * p.q_bs + qpos * p.q_rs + hq * p.q_hs + h32 * 8;
+  auto scale_q = [&] {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
+    if (p.negate_q) {
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      u32x4 raw = *reinterpret_cast<const u32x4*>(qrow + ks * 16);
-      if (p.negate_q) raw ^= 0x80008000u;
-      qf[ks] = __builtin_bit_cast(bf16x8, raw);
+      for (int ks = 0; ks < 8; ++ks)
+        qf[ks] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, qf[ks]) ^ 0x80008000u);
     }
-  }
+  };
 
-  // ---------------------------------------------------------------- loader addressing
-  // thread handles 16-byte chunk (tid % 16) of tile rows tid/16 + (NT/16)*pass
-  const int ld_chunk = tid & 15;
-  const int ld_row0 = tid >> 4;
-  // Row gather addresses: uniform base pointer + per-lane 32-bit byte offset whenever every row of
-  // the (batch, kv head) slice lies within 4 GiB of its base (checked on the host), which keeps
-  // the address arithmetic to a couple of 24-bit multiplies per tile.
+  // ---------------------------------------------------------------- loader: HBM rows -> LDS
+  // One global_load_lds_dwordx4 moves a 4-row group: lane L fetches 16 bytes of row L/16 and the
+  // hardware writes the 64 x 16 bytes to consecutive LDS addresses from M0, so lane L has to
+  // fetch the chunk that belongs into slot L%16 of its row.  No VGPR staging and no LDS store
+  // instructions; rows past the last key are clamped to it.
+  constexpr int GROUPS_PER_WAVE = (BN / 4) / NW;
+  static_assert((BN / 4) % NW == 0, "tile groups must split evenly over the wavefronts");
   const char* kbase = reinterpret_cast<const char*>(p.k + batch * p.k_bs + kvh * p.k_hs);
   const char* vbase = reinterpret_cast<const char*>(p.v + batch * p.v_bs + kvh * p.v_hs);
-  u32x4 kst[LD_PASSES], vst[LD_PASSES];
-  const int ld_koff = ld_row0 * KSTRIDE + ld_chunk * 16;
-  const int ld_voff = VBASE + ld_row0 * VSTRIDE + ld_chunk * 16;
+  const int ld_row = lane >> 4;                                  // row of the group this lane fetches
+  const uint32_t ld_col = (((lane & 15) ^ (4 * ld_row)) << 4);   // byte column it fetches
   const uint32_t k_rs_b = p.k_rs_bytes, v_rs_b = p.v_rs_bytes;
-  const uint32_t ld_col = ld_chunk * 16;
-
-  auto load_k = [&](int tile) {
-    const int kb = kt_lo + tile * BN;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  auto load_tile = [&](const char* base, uint32_t rs_b, int tile, int lds_off) {
 #pragma unroll
-    for (int ps = 0; ps < LD_PASSES; ++ps) {
-      int tk = im_min(kb + ld_row0 + ps * (NT / 16), nk - 1);
-      uint32_t pos = map.kpos(tk);
-      if (p.small_offsets)
-        kst[ps] = *reinterpret_cast<const u32x4*>(kbase + (__umul24(pos, k_rs_b) + ld_col));
-      else
-        kst[ps] = *reinterpret_cast<const u32x4*>(kbase + ((int64_t)pos * p.k_rs * 2 + ld_col));
+    for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
+      const int grp = wave * GROUPS_PER_WAVE + gi;
+      const int tk = im_min(kt_lo + tile * BN + 4 * grp + ld_row, nk - 1);
+      const uint32_t pos = map.kpos(tk);
+      dma_group(base + ((uint64_t)pos * rs_b + ld_col), lds_base + lds_off + grp * GROUP_STRIDE);  // one 32x32+64 mad
     }
   };
-  auto load_v = [&](int tile) {
-    const int kb = kt_lo + tile * BN;
-#pragma unroll
-    for (int ps = 0; ps < LD_PASSES; ++ps) {
-      int tk = im_min(kb + ld_row0 + ps * (NT / 16), nk - 1);
-      uint32_t pos = map.kpos(tk);
-      if (p.small_offsets)
-        vst[ps] = *reinterpret_cast<const u32x4*>(vbase + (__umul24(pos, v_rs_b) + ld_col));
-      else
-        vst[ps] = *reinterpret_cast<const u32x4*>(vbase + ((int64_t)pos * p.v_rs * 2 + ld_col));
-    }
-  };
-  auto store_k = [&](int kbuf_off) {
-#pragma unroll
-    for (int ps = 0; ps < LD_PASSES; ++ps)
-      *reinterpret_cast<u32x4*>(smem + kbuf_off + ld_koff + ps * (NT / 16) * KSTRIDE) = kst[ps];
-  };
-  auto store_v = [&](int vbuf_off) {
-#pragma unroll
-    for (int ps = 0; ps < LD_PASSES; ++ps)
-      *reinterpret_cast<u32x4*>(smem + vbuf_off + ld_voff + ps * (NT / 16) * VSTRIDE) = vst[ps];
-  };
+  auto load_k = [&](int tile, int kbuf_off) { load_tile(kbase, k_rs_b, tile, kbuf_off); };
+  auto load_v = [&](int tile, int vbuf_off) { load_tile(vbase, v_rs_b, tile, VBASE + vbuf_off); };
 
   // K operand (A of S^T = K Q^T): lane reads 16 bytes of key row l32 at head dims 16*ks + 8*h32
-  const int klane = l32 * KSTRIDE + h32 * 16;
+  int kaddr[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks)
+    kaddr[ks] = (l32 >> 2) * GROUP_STRIDE + (l32 & 3) * 256 + (((2 * ks + h32) ^ (4 * (l32 & 3))) << 4);
   // V^T operand (A of O^T = V^T P^T) through transposing reads.  Within each group of 16 lanes,
   // lane i supplies the address of 4 head dims (4*(i%4)..) of key row i/4 and receives head dim i
   // of those 4 key rows.  Lane groups 0/1 take head dims 0-15/16-31 of a 32-dim block, the upper
-  // 32 lanes the key rows 4..7 of each group of 8.
-  const int vlane = VBASE + (4 * h32 + ((lane & 15) >> 2)) * VSTRIDE + 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+  // 32 lanes the key rows 4..7 of each 8 (the next 4-row group).  vaddr[db]: 32-dim block db.
+  int vaddr[4];
+  {
+    const int i16 = lane & 15, g2 = (lane >> 4) & 1, ri = i16 >> 2;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+      vaddr[db] = VBASE + h32 * GROUP_STRIDE + ri * 256 + (((4 * db + 2 * g2 + ((i16 & 3) >> 1)) ^ (4 * ri)) << 4) +
+                  8 * (i16 & 1);
+  }
 
   // ---------------------------------------------------------------- running softmax state
   floatx16 oacc[4];
@@ -230,33 +245,34 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   for (int db = 0; db < 4; ++db)
 #pragma unroll
     for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
-  floatx16 s0, s1;  // scores of two consecutive 32-key blocks
-  float m_run = -INFINITY;  // reference maximum of the exponentials (raw score units)
-  float mc = 0.f;           // m_run * c, 0 while m_run is still -inf
+  floatx16 s0, s1;  // raw scores q.k of two consecutive 32-key blocks
+  // Exponent reference of this lane's query.  Weights are exp2(score * c - mref) and numerator and
+  // denominator always share mref, so any value gives the exact softmax as long as nothing
+  // overflows or underflows.  fp32 and bf16 both span 2^+-126, so mref stays 0 (and costs nothing)
+  // for every query whose scores stay within +-60 of it; it is re-centred on a block's maximum
+  // when that maximum leaves this band upwards, or downwards before anything was accumulated.
+  float mref = 0.f;
   float l_run = 0.f;
-  const float c = p.scale_log2;
+  const float c = p.scale_log2;  // |softmax_scale| * log2(e)
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
-  const float gap = p.rescale_gap;
 
   // operand reads; koff / voff are byte offsets of (buffer, 32-key block) in LDS
-  auto kread = [&](int koff, int ks) {
-    return *reinterpret_cast<const bf16x8*>(smem + koff + klane + ks * 32);
-  };
+  auto kread = [&](int koff, int ks) { return *reinterpret_cast<const bf16x8*>(smem + koff + kaddr[ks]); };
   auto vread = [&](int voff, int j) {  // j = 4 * t + db: keys 16t..16t+15 of the block, head dims 32db..
-    const int off = (j >> 2) * 16 * VSTRIDE + (j & 3) * 64;
+    const int off = (j >> 2) * 4 * GROUP_STRIDE;
     bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (__attribute__((address_space(3))) bf16x4*)(smem + voff + vlane + off));
+        (__attribute__((address_space(3))) bf16x4*)(smem + voff + vaddr[j & 3] + off));
     bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (__attribute__((address_space(3))) bf16x4*)(smem + voff + vlane + off + 8 * VSTRIDE));
+        (__attribute__((address_space(3))) bf16x4*)(smem + voff + vaddr[j & 3] + off + 2 * GROUP_STRIDE));
     return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
   };
+
   auto zero16 = [] {
     floatx16 z;
 #pragma unroll
     for (int e = 0; e < 16; ++e) z[e] = 0.f;
     return z;
   };
-
   // ----- unscheduled pieces, used at the edges of a wavefront's key range
   auto qk_block = [&](floatx16& acc, int koff) {
     acc = zero16();
@@ -271,15 +287,28 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
       if (key < lo_l || key > hi_l) s[e] = -INFINITY;
     }
   };
-  // The running maximum only moves when some query's block maximum exceeds it by more than
-  // `gap`; until then the exponentials just grow up to 2^8, which fp32/bf16 hold easily.
-  auto raise_max = [&](float mx) {
-    if (__builtin_amdgcn_ballot_w64(mx > m_run + gap) != 0) {
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-      m_run = m_new;
-      mc = m_use * c;
+  auto block_max = [&](const floatx16& s) {
+    float m0 = fmaxf(fmaxf(s[0], s[1]), s[2]);
+    m0 = fmaxf(fmaxf(m0, s[3]), s[4]);
+    m0 = fmaxf(fmaxf(m0, s[5]), s[6]);
+    float m1 = fmaxf(fmaxf(s[8], s[9]), s[10]);
+    m1 = fmaxf(fmaxf(m1, s[11]), s[12]);
+    m1 = fmaxf(fmaxf(m1, s[13]), s[14]);
+    return lane_xor32_max(fmaxf(fmaxf(m0, s[7]), fmaxf(m1, s[15])));
+  };
+  // What can happen to a freshly computed block of raw scores q.k before it is exponentiated as
+  // exp2(score * c - mref); all of it is rare.  `mx` is the block maximum of the raw scores.
+  auto settle = [&](floatx16& nxt, float mx, bool masked, int kb32) {
+    if (masked) {  // block cut by a bound: mask in place, then redo the maximum
+      mask_block(nxt, kb32);
+      mx = block_max(nxt);
+    }
+    const float mxs = __builtin_fmaf(mx, c, -mref);  // block maximum in exponent units
+    const bool need = mxs > 60.f || (l_run == 0.f && mxs < -60.f && mxs > -INFINITY);
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {
+      const float delta = need ? mxs : 0.f;
+      const float alpha = l_run == 0.f ? 1.f : __builtin_amdgcn_exp2f(-delta);
+      mref += delta;
       l_run *= alpha;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
@@ -287,160 +316,163 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
         for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
     }
   };
-  // ----- loader work of one tile iteration: put the rows fetched during the previous iteration
-  // (K(i+2), V(i+1), waiting in registers) into the LDS buffers of K(i-1) and V(i-1), then start
-  // fetching K(i+3) and V(i+2).  Rows past the end are clamped to the last key, so the tail
-  // iterations just re-read one cached row instead of branching.
-  auto loader = [&](int i, int kdst, int vdst) {
-    store_k(kdst);
-    store_v(vdst);
-    load_k(i + 3);
-    load_v(i + 2);
-  };
 
   // ----- hand-scheduled step: QK^T of the next key block (8 MFMAs) and PV of the current one
-  // (8 MFMAs) with the softmax VALU work of the current block spread between them.  One "slot"
-  // is one MFMA.  LDS operands are fetched a whole phase (8 slots) ahead: the V^T operands of
-  // this step's PV during its QK^T slots, the K operands of the NEXT step's QK^T during this
-  // step's PV slots (ka lives across steps and across the tile barrier: the K tile it reads was
-  // made visible by an earlier barrier and is not overwritten before the next one), so each
-  // phase opens with a single wait.  The exponentials are cut into 8 units of one bf16 pair and
-  // run through a 3-stage pipeline (scale, exp2, pack + row sum) one slot apart, so that no VALU
-  // instruction waits for the one issued just before it; P^T half 0 is complete at slot 7, half
-  // 1 at slot 11.  The first step of a tile also carries the tile's loader work in slots 12..15,
-  // where the VALU is otherwise idle.  sched_barrier keeps the compiler from regrouping.
+  // (8 MFMAs) with the softmax VALU work spread between them.  One "slot" is one MFMA.  LDS
+  // operands are fetched a whole phase (8 slots) ahead: the V^T operands of this step's PV during
+  // its QK^T slots, the K operands of the NEXT step's QK^T during this step's PV slots (ka lives
+  // across steps and across the tile barrier: the K tile it reads was made visible by an earlier
+  // barrier and is not overwritten before the next one).  The exponentials of the current block
+  // run one bf16 pair per slot in slots 0..7, the packing + row sums one slot later; the maximum
+  // of the next block is taken in the PV slots once its MFMA chain has drained.
+  // sched_barrier keeps the compiler from regrouping the slots.
   bf16x8 ka[8];
-  auto steady = [&](const floatx16& s, floatx16& n, int koff_next, int voff, auto with_loader, int i,
-                    int kdst, int vdst) {
+  auto steady = [&](const floatx16& s, floatx16& n, int koff_next, int voff, bool mask_next, int kb32_next) {
     bf16x8 va[8], pb[2];
-    float mx0, mx1;
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): ka[] has landed
-#pragma unroll
-    for (int g = 0; g < 2; ++g) {
-      va[g] = vread(voff, g);
-      n = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[g], qf[g], g == 0 ? zero16() : n, 0, 0, 0);
-      const int e0 = 8 * g;
-      float m = fmaxf(fmaxf(s[e0], s[e0 + 1]), s[e0 + 2]);
-      m = fmaxf(fmaxf(m, s[e0 + 3]), s[e0 + 4]);
-      m = fmaxf(fmaxf(m, s[e0 + 5]), s[e0 + 6]);
-      m = fmaxf(m, s[e0 + 7]);
-      if (g == 0) mx0 = m;
-      else mx1 = m;
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    raise_max(lane_xor32_max(fmaxf(mx0, mx1)));
-    float rs = 0.f;
-    float fx[8][2], px[8][2];
-    auto stage_f = [&](int u) {
-      fx[u][0] = __builtin_fmaf(s[2 * u], c, -mc);
-      fx[u][1] = __builtin_fmaf(s[2 * u + 1], c, -mc);
-    };
+    float rs[2] = {0.f, 0.f};
+    float px[8][2];
     auto stage_e = [&](int u) {
-      px[u][0] = __builtin_amdgcn_exp2f(fx[u][0]);
-      px[u][1] = __builtin_amdgcn_exp2f(fx[u][1]);
+      px[u][0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u], c, -mref));
+      px[u][1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u + 1], c, -mref));
     };
     auto stage_c = [&](int u) {
       floatx2 f = {px[u][0], px[u][1]};
       bf16x2 h = __builtin_convertvector(f, bf16x2);
-      rs = __builtin_amdgcn_fdot2_f32_bf16(h, ones2, rs, false);  // sums what PV will multiply
+      rs[u & 1] = __builtin_amdgcn_fdot2_f32_bf16(h, ones2, rs[u & 1], false);  // sums what PV multiplies
       pb[u >> 2][2 * (u & 3)] = h[0];
       pb[u >> 2][2 * (u & 3) + 1] = h[1];
     };
-    auto valu_slot = [&](int k) {  // slot k: scale unit k-2, exp2 unit k-3, pack unit k-4
-      if (k - 2 >= 0 && k - 2 < 8) stage_f(k - 2);
-      if (k - 3 >= 0 && k - 3 < 8) stage_e(k - 3);
-      if (k - 4 >= 0 && k - 4 < 8) stage_c(k - 4);
+    // exp2 of pair u is issued in slot e_slot(u), packed one slot later: pairs 0-3 (P^T half 0,
+    // needed from slot 8) in every other QK^T slot, pairs 4-7 (half 1, needed from slot 12) in
+    // slots 7..10, the maximum of the new block in slots 12..15.  Both phases then carry about
+    // the same VALU load per MFMA, which matters because the two wavefronts of a SIMD tend to
+    // be in the same phase.
+    auto valu_slot = [&](int k) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int es = u < 4 ? 2 * u : u + 3;
+        if (es == k) stage_e(u);
+        if (es + 1 == k) stage_c(u);
+      }
     };
 #pragma unroll
-    for (int g = 2; g < 8; ++g) {
+    for (int g = 0; g < 8; ++g) {
       va[g] = vread(voff, g);
-      n = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[g], qf[g], n, 0, 0, 0);
+      n = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[g], qf[g], g == 0 ? zero16() : n, 0, 0, 0);
       valu_slot(g);
       __builtin_amdgcn_sched_barrier(0);
     }
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): va[] has landed
+    float m0, m1;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       ka[j] = kread(koff_next, j);
       oacc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[j], pb[j >> 2], oacc[j & 3], 0, 0, 0);
       valu_slot(8 + j);
-
+      if (j == 4) m0 = fmaxf(fmaxf(n[0], n[1]), fmaxf(n[2], n[3]));
+      if (j == 5) m0 = fmaxf(fmaxf(m0, n[4]), fmaxf(n[5], fmaxf(n[6], n[7])));
+      if (j == 6) m1 = fmaxf(fmaxf(n[8], n[9]), fmaxf(n[10], n[11]));
+      if (j == 7) m1 = fmaxf(fmaxf(m1, n[12]), fmaxf(n[13], fmaxf(n[14], n[15])));
       __builtin_amdgcn_sched_barrier(0);
     }
-    l_run += rs;
+    l_run += rs[0] + rs[1];
+    settle(n, lane_xor32_max(fmaxf(m0, m1)), mask_next, kb32_next);
   };
 
   // Step j: softmax + PV of key block j (scores in `cur`, V rows at voff) and QK^T of key block
   // j+1 into `nxt` (its K rows at koff; those of block j+2 at koff_next).  A wavefront runs the
   // steps jq..jp with jq = bw_lo - 1: in step jq only the QK^T half matters, so its scores are
-  // preset to -inf (weights 0, the maximum stays -inf); in step jp the QK^T half computes a block
-  // nobody reads.  That keeps one code path through the accumulators.
+  // preset to -inf (weights 0); in step jp the QK^T half computes a block nobody reads (masked
+  // to -inf so that it cannot move the reference).  That keeps one code path through the
+  // accumulators.  Blocks not inside [f_lo, f_hi] get the per-element mask.
   const int jq = bw_lo - 1, jp = bw_hi;
+  auto needs_mask = [&](int j) {
+    const int kb32 = kt_lo + 32 * j;
+    return j >= jp + 1 || kb32 < f_lo || kb32 + 31 > f_hi;
+  };
   auto step = [&](int j, floatx16& cur, floatx16& nxt, int koff, int koff_next, int voff, auto with_loader,
                   int i, int kdst, int vdst) {
-    if (decltype(with_loader)::value) loader(i, kdst, vdst);
+    if (decltype(with_loader)::value) {
+      load_k(i + 3, kdst);
+      load_v(i + 2, vdst);
+    }
     if (j < jq || j > jp) return;
-    const int kb32 = kt_lo + 32 * j;
     if (j == jq) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) cur[e] = -INFINITY;
 #pragma unroll
       for (int g = 0; g < 8; ++g) ka[g] = kread(koff, g);
-    } else if (kb32 < f_lo || kb32 + 31 > f_hi) {
-      mask_block(cur, kb32);
     }
-    steady(cur, nxt, koff_next, voff, with_loader, i, kdst, vdst);
+    steady(cur, nxt, koff_next, voff, needs_mask(j + 1), kt_lo + 32 * (j + 1));
   };
 
   // ---------------------------------------------------------------- main loop
-  // At the top of iteration i the LDS holds K(i), K(i+1) and V(i), and the staging registers hold
-  // (or are receiving) K(i+2) and V(i+1).  During the iteration those go into the buffers of
-  // K(i-1) and V(i-1), which no wavefront reads after the barrier that opened iteration i, and
-  // the fetch of K(i+3) and V(i+2) starts: every global load has a whole iteration to arrive.
-  load_k(0);
-  load_v(0);
-  store_k(0);
-  store_v(0);
-  load_k(1);
-  store_k(KTILE);
-  load_k(2);
-  load_v(1);
-  __syncthreads();
+  // K tile t lives in ring slot t % 4, V tile t in slot t % 3.  At the top of iteration i the LDS
+  // holds K(i), K(i+1), V(i); K(i+2) and V(i+1) were requested during iteration i-1 and may still
+  // be in flight.  Iteration i requests K(i+3) and V(i+2) into the slots of K(i-1) and V(i-1),
+  // which no wavefront reads after the barrier that opened iteration i.  The barrier that opens
+  // iteration i+1 only waits for the older requests, so every row has a whole iteration to arrive.
+  constexpr int PER_TILE = 2 * GROUPS_PER_WAVE;  // loads per wavefront per iteration (K + V)
+  load_k(0, 0);
+  load_v(0, 0);
+  load_k(1, KTILE);
+  load_k(2, 2 * KTILE);
+  load_v(1, VTILE);
+  {
+    // Q goes through the same in-order load counter as the tile requests above, so by the time
+    // it can be scaled the first tiles have landed as well: one memory latency for the prologue.
+    const uint16_t* qrow = p.q + batch * p.q_bs + qpos * p.q_rs + hq * p.q_hs + h32 * 8;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + ks * 16);
+  }
+  scale_q();
+  tile_barrier<PER_TILE>();
   if (jq < 0 && jp >= 0) {
     qk_block(s0, 0);
+    settle(s0, block_max(s0), needs_mask(0), kt_lo);
 #pragma unroll
-    for (int g = 0; g < 8; ++g) ka[g] = kread(32 * KSTRIDE, g);
+    for (int g = 0; g < 8; ++g) ka[g] = kread(BLOCK32, g);
   }
-  int kcur = 0, knext = KTILE, knext2 = 2 * KTILE;
+  int k0 = 0, k1 = KTILE, k2 = 2 * KTILE, k3 = 3 * KTILE;  // slots of K(i), K(i+1), K(i+2), K(i+3)
+  int v0 = 0, v1 = VTILE, v2 = 2 * VTILE;                  // slots of V(i), V(i+1), V(i+2)
   for (int i = 0; i < ntiles; ++i) {
-    __syncthreads();
-    const int vcur = (i & 1) * VTILE;
-    step(2 * i, s0, s1, kcur + 32 * KSTRIDE, knext, vcur, ic<1>{}, i, knext2, VTILE - vcur);
-    step(2 * i + 1, s1, s0, knext, knext + 32 * KSTRIDE, vcur + 32 * VSTRIDE, ic<0>{}, i, 0, 0);
-    const int t = kcur;
-    kcur = knext;
-    knext = knext2;
-    knext2 = t;
+    if (i > 0) tile_barrier<PER_TILE>();
+    step(2 * i, s0, s1, k0 + BLOCK32, k1, v0, ic<1>{}, i, k3, v2);
+    step(2 * i + 1, s1, s0, k1, k1 + BLOCK32, v0 + BLOCK32, ic<0>{}, i, 0, 0);
+    const int tk = k0;
+    k0 = k1; k1 = k2; k2 = k3; k3 = tk;
+    const int tv = v0;
+    v0 = v1; v1 = v2; v2 = tv;
   }
 
   // ---------------------------------------------------------------- normalise and scatter-store
-  if (!wave_active) return;
+  if (!wave_active) continue;
   const float l_tot = lane_xor32_sum(l_run);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (row_valid) {
-    uint16_t* orow = p.o + batch * p.o_bs + qpos * p.o_rs + hq * p.o_hs + 4 * h32;
+  // Lane l and lane l+32 hold the same query: per 16 head dims the lower lane has dims 0-3 and
+  // 8-11, the upper one 4-7 and 12-15.  One permlane32 swap per register pair turns that into
+  // dims 0-7 / 8-15, so each lane writes 16 contiguous bytes.
+  uint16_t* orow = p.o + batch * p.o_bs + qpos * p.o_rs + hq * p.o_hs + 8 * h32;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+  for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        floatx2 f0 = {oacc[db][4 * g] * inv, oacc[db][4 * g + 1] * inv};
-        floatx2 f1 = {oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv};
-        bf16x2 b0 = __builtin_convertvector(f0, bf16x2);
-        bf16x2 b1 = __builtin_convertvector(f1, bf16x2);
-        u32x2 pk = {__builtin_bit_cast(uint32_t, b0), __builtin_bit_cast(uint32_t, b1)};
-        *reinterpret_cast<u32x2*>(orow + 32 * db + 8 * g) = pk;
+    for (int g2 = 0; g2 < 2; ++g2) {
+      uint32_t w[4];
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          const int e = 8 * g2 + 4 * half + 2 * k;
+          floatx2 f = {oacc[db][e] * inv, oacc[db][e + 1] * inv};
+          w[2 * half + k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+        }
+      auto r0 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+      auto r1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+      if (row_valid) {
+        u32x4 pk = {r0[0], r1[0], r0[1], r1[1]};
+        *reinterpret_cast<u32x4*>(orow + 32 * db + 16 * g2) = pk;
       }
-  }
+    }
+  }  // work items
 }
 
 }  // namespace intra

@@ -34,7 +34,7 @@ def test_plan_headline(lib):
     rc, p = _plan(lib, 0, 0, 1, 32768, 32, 8, 8, 576)
     assert rc == 0
     assert (p.heads_per_block, p.waves, p.pos_per_block) == (4, 8, 64)
-    assert (p.n_sets, p.n_mblocks, p.grid) == (8, 64, 4096)
+    assert (p.n_sets, p.n_mblocks, p.work_items, p.grid) == (8, 64, 4096, 4096)
     assert p.pairs_per_head == 67125248 and 0 < p.lds_bytes <= 160 * 1024
 
 
