@@ -22,7 +22,7 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU; AMD publishes it as 2.5 PFLOP/s dense
 # HBM bytes per launch at S=32768 measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/); None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {32768: 971e6}
 
 
 def main():

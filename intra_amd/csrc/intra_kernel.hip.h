@@ -14,17 +14,20 @@
 //  * O^T = V^T P^T: P^T is the softmax output still in registers (packed to bf16, no LDS round
 //    trip); V^T comes from ds_read_b64_tr_b16 transposing reads of the row-major V tile.
 //  * Software pipeline in steps of 32 keys: in step j a wavefront issues the 8 QK^T MFMAs of key
-//    block j+1 next to the softmax VALU work of block j, then the 8 PV MFMAs of block j, with
-//    all LDS operand reads issued two MFMAs ahead.  K therefore runs up to one tile ahead of V
-//    in LDS: three K buffers, two V buffers, one barrier per 64-key tile.
-//  * K/V rows are gathered from HBM with 16-byte loads, 16 lanes per 256-byte row, staged in
-//    registers during the iteration and written to the free LDS buffers at its end.  LDS rows
-//    are padded (K: 272 B, V: 320 B) so that the row-per-lane K reads and the 4-row transposing
-//    V reads both spread over all 64 banks with plain base + immediate addressing.
-//  * The running maximum is only raised (and O rescaled) when a tile's maximum exceeds it by
-//    more than 2^8 in the exponent; softmax weights are exact after the final normalisation
-//    because numerator and denominator share the reference maximum.
-//  * Tiles outside a wavefront's key range are skipped; only tiles cut by a bound are masked.
+//    block j+1 and the 8 PV MFMAs of block j, with the softmax VALU work of block j spread over
+//    both phases and every LDS operand read issued a whole phase (8 MFMAs) ahead.
+//  * K/V rows are gathered from HBM straight into LDS (global_load_lds_dwordx4, 16 lanes per
+//    256-byte row, no register staging), three tiles ahead for K and two for V; one barrier per
+//    64-key tile, which only waits for the requests of the previous iteration.  An LDS tile is
+//    16 groups of 4 rows with an XOR chunk swizzle inside the group and 16 bytes of padding
+//    between groups, so the row-per-lane K reads and the 4-row transposing V reads are both free
+//    of bank conflicts.
+//  * The softmax reference stays 0 (weights exp2(score*c), exact after normalisation because
+//    numerator and denominator share it) unless a block maximum leaves the +-60 exponent band;
+//    then the query is re-centred and O rescaled.  No per-block rescale in the common case.
+//  * Blocks outside a wavefront's key range are skipped; only blocks cut by a bound are masked.
+//  * The grid is persistent (about one workgroup per CU); work items are dealt per XCD so that
+//    one (batch, kv head, set) stays in one XCD's L2, in an order that balances causal triangles.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
