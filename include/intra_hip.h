@@ -69,15 +69,16 @@ int intra_version(void);
  * launchers (csrc/flash_attn/src/flash_fwd_launch_template.h:401-565, flash_api.cpp:408-411,
  * 611-612, 703-714). */
 typedef struct IntraPlan {
-  int kind;            /* internal kernel kind 0..4 */
-  int heads_per_block; /* query heads of one kv head packed into a workgroup */
-  int waves;           /* wavefronts per workgroup */
-  int pos_per_block;   /* in-set queries per workgroup */
-  int n_sets;          /* sets per (batch, kv head) */
-  int n_mblocks;       /* row blocks of the largest set */
-  int work_items;      /* row blocks to process (a multiple of 8: padded per XCD) */
+  int kind;            /* internal pattern kind 0..4 */
+  int heads_per_block; /* query heads of one kv head packed into a workgroup (main launch) */
+  int waves;           /* wavefronts per workgroup (main launch) */
+  int pos_per_block;   /* in-set queries per workgroup (main launch) */
+  int n_sets;          /* sets per (batch, kv head) (main launch) */
+  int n_mblocks;       /* row blocks of the largest set (main launch) */
+  int work_items;      /* row blocks to process, all launches (a multiple of 8: padded per XCD) */
   int grid;            /* upper bound of workgroups launched: min(work_items, CUs of the device) */
   int lds_bytes;       /* LDS per workgroup */
+  int launches;        /* kernel launches per call: 1, or 2 for image gather0 (grid rows, text rows) */
   int64_t pairs_per_head; /* unmasked (query, key) pairs per query head and batch */
 } IntraPlan;
 
@@ -88,7 +89,7 @@ int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, 
 /* Walks the exact set / row-block / wavefront / 32-key-block decomposition the kernel uses
  * (same index maps and block classification, compiled for the host) and adds 1 to
  * count[q_pos * S + k_pos] for every score the kernel would compute and keep.  `count` is an
- * S*S byte array the caller zeroed.  heads_per_block / waves <= 0 pick the library default. */
+ * S*S byte array the caller zeroed.  heads_per_block <= 0 means 1; waves must be 8 or <= 0. */
 int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int heads_per_block,
                      int waves, uint8_t* count);
 

@@ -14,7 +14,8 @@ _i64x3 = ctypes.c_int64 * 3
 class IntraPlan(ctypes.Structure):
     _fields_ = [("kind", ctypes.c_int), ("heads_per_block", ctypes.c_int), ("waves", ctypes.c_int),
                 ("pos_per_block", ctypes.c_int), ("n_sets", ctypes.c_int), ("n_mblocks", ctypes.c_int),
-                ("work_items", ctypes.c_int), ("grid", ctypes.c_int), ("lds_bytes", ctypes.c_int), ("pairs_per_head", ctypes.c_int64)]
+                ("work_items", ctypes.c_int), ("grid", ctypes.c_int), ("lds_bytes", ctypes.c_int), ("launches", ctypes.c_int),
+                ("pairs_per_head", ctypes.c_int64)]
 
 
 _FWD_ARGS = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 4 + \

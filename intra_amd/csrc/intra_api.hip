@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <type_traits>
+
 #include "../../include/intra_hip.h"
 #include "intra_kernel.hip.h"
 
@@ -39,7 +41,7 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   r->S = S;
   r->H = H;
   r->Hkv = Hkv;
-  r->geom = IntraGeom{S, 1, 64, 16, 8};
+  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1};
   if (domain == 0) {
     if (pattern == INTRA_LLM_SCATTER || pattern == INTRA_LLM_GATHER1) {
       if (arg0 < 1) return fail(INTRA_ERR_INVALID, "group_num must be >= 1 (got %d)", arg0);
@@ -73,60 +75,117 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   return INTRA_OK;
 }
 
-// Workgroup shape: HP query heads of one kv head share a workgroup.  Gather0 sets are single
-// 64-query blocks, so its workgroups shrink with HP; the other patterns always run 8 wavefronts.
-void pick_shape(int kind, int ratio, int* hp, int* nw) {
-  int h = ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1);
-  *hp = h;
-  *nw = kind == KIND_IMG_GATHER0 ? 2 * h : 8;
+// One kernel launch: an index map, its geometry and the workgroup shape (HP query heads of one kv
+// head share a workgroup of NW wavefronts, so a row block has NW * 32 / HP in-set queries).
+enum MapId : int { MAP_LLM_SCATTER, MAP_LLM_GATHER1, MAP_LLM_WINDOW, MAP_IMG_SCATTER, MAP_IMG_PATCH };
+struct Phase {
+  int map;
+  IntraGeom geom;
+  int hp, nw;
+};
+
+int default_hp(int ratio) { return ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1); }
+
+// Every pattern is one launch of 8-wavefront workgroups, except image gather0: its grid queries
+// run as sets of `pg` neighbouring 8x8 patches (as many as fit into a row block), its text
+// queries - which see what the scatter pattern shows them - as text-only scatter sets, whose
+// 64-query chunks get workgroups of 2 * HP wavefronts.
+int phases_for(const Request& r, int hp, Phase ph[2]) {
+  ph[0].geom = r.geom;
+  ph[0].hp = hp;
+  ph[0].nw = 8;
+  switch (r.kind) {
+    case KIND_LLM_SCATTER: ph[0].map = MAP_LLM_SCATTER; return 1;
+    case KIND_LLM_GATHER1: ph[0].map = MAP_LLM_GATHER1; return 1;
+    case KIND_LLM_WINDOW: ph[0].map = MAP_LLM_WINDOW; return 1;
+    case KIND_IMG_SCATTER: ph[0].map = MAP_IMG_SCATTER; return 1;
+    default: break;
+  }
+  const int np = r.geom.width / 8;
+  int pg = im_max(1, (8 * 32 / hp) / 64);
+  while (np % pg != 0) --pg;
+  ph[0].map = MAP_IMG_PATCH;
+  ph[0].geom.pg = pg;
+  ph[1] = ph[0];
+  ph[1].map = MAP_IMG_SCATTER;
+  ph[1].geom.text_only = 1;
+  ph[1].nw = 2 * hp;
+  return 2;
 }
 
-bool shape_ok(int kind, int hp, int nw) {
-  if (hp != 1 && hp != 2 && hp != 4) return false;
-  if (kind == KIND_IMG_GATHER0) return nw == 2 * hp;
-  return nw == 8;
+struct PhaseDims {
+  int pos, n_sets, n_mblocks, hgroups, n_pairs, work_items;
+};
+
+template <class MAP>
+PhaseDims dims_of(const Request& r, const Phase& ph) {
+  PhaseDims d;
+  d.pos = ph.nw * 32 / ph.hp;
+  d.n_sets = MAP::num_sets(ph.geom);
+  d.n_mblocks = (MAP::max_nq(ph.geom) + d.pos - 1) / d.pos;
+  d.hgroups = (r.H / r.Hkv) / ph.hp;
+  const int64_t n_pairs = (int64_t)r.B * r.Hkv * d.n_sets;
+  const int64_t items = 8 * ((n_pairs + 7) / 8) * d.hgroups * d.n_mblocks;
+  d.n_pairs = n_pairs > 0x7fffffff ? -1 : (int)n_pairs;
+  d.work_items = items > 0x7fffffff ? -1 : (int)items;
+  return d;
 }
 
 template <class MAP>
-void fill_plan(const Request& r, int hp, int nw, IntraPlan* plan) {
-  const int pos = nw * 32 / hp;
-  plan->kind = r.kind;
-  plan->heads_per_block = hp;
-  plan->waves = nw;
-  plan->pos_per_block = pos;
-  plan->n_sets = MAP::num_sets(r.geom);
-  plan->n_mblocks = (MAP::max_nq(r.geom) + pos - 1) / pos;
-  const int hgroups = (r.H / r.Hkv) / hp;
-  const int64_t n_pairs = (int64_t)r.B * r.Hkv * plan->n_sets;
-  const int64_t items = 8 * ((n_pairs + 7) / 8) * hgroups * plan->n_mblocks;
-  plan->work_items = items > 0x7fffffff ? -1 : (int)items;
-  plan->grid = plan->work_items;  // upper bound; a launch uses min(work_items, 8 * (CUs / 8))
-  plan->lds_bytes = intra::LDS_BYTES;
+int64_t pairs_of(const IntraGeom& ge) {
   int64_t pairs = 0;
-  for (int set = 0; set < plan->n_sets; ++set) {
-    MAP map(r.geom, set);
-    const int nq = map.nq(), nk = map.nk();
+  const int n_sets = MAP::num_sets(ge);
+  for (int set = 0; set < n_sets; ++set) {
+    MAP map(ge, set);
+    const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
     for (int tq = 0; tq < nq; ++tq) {
-      int hi = im_min(map.khi(tq), nk - 1);
-      int lo = map.klo(tq);
-      if (hi >= lo) pairs += hi - lo + 1;
+      const int hi = im_min(map.khi(tq), nk - 1);
+      const int lo = im_max(map.klo(tq), kpre);
+      pairs += kpre + (hi >= lo ? hi - lo + 1 : 0);
     }
   }
+  return pairs;
+}
+
+template <template <class> class F, class... A>
+auto by_map(int map, A&&... a) {
+  switch (map) {
+    case MAP_LLM_SCATTER: return F<MapLlmScatter>::go(a...);
+    case MAP_LLM_GATHER1: return F<MapLlmGather1>::go(a...);
+    case MAP_LLM_WINDOW: return F<MapLlmWindow>::go(a...);
+    case MAP_IMG_SCATTER: return F<MapImgScatter>::go(a...);
+    default: return F<MapImgPatch>::go(a...);
+  }
+}
+template <class MAP> struct DimsOf { static PhaseDims go(const Request& r, const Phase& ph) { return dims_of<MAP>(r, ph); } };
+template <class MAP> struct PairsOf { static int64_t go(const IntraGeom& ge) { return pairs_of<MAP>(ge); } };
+
+// The plan describes the first (main) launch; work items and pairs are summed over all launches.
+void plan_for(const Request& r, int hp, IntraPlan* plan) {
+  Phase ph[2];
+  const int n = phases_for(r, hp, ph);
+  const PhaseDims d = by_map<DimsOf>(ph[0].map, r, ph[0]);
+  plan->kind = r.kind;
+  plan->heads_per_block = ph[0].hp;
+  plan->waves = ph[0].nw;
+  plan->pos_per_block = d.pos;
+  plan->n_sets = d.n_sets;
+  plan->n_mblocks = d.n_mblocks;
+  plan->launches = n;
+  plan->lds_bytes = intra::LDS_BYTES;
+  int64_t items = 0, pairs = 0;
+  for (int i = 0; i < n; ++i) {
+    const PhaseDims di = by_map<DimsOf>(ph[i].map, r, ph[i]);
+    items = (di.work_items < 0 || items < 0) ? -1 : items + di.work_items;
+    pairs += by_map<PairsOf>(ph[i].map, ph[i].geom);
+  }
+  plan->work_items = items > 0x7fffffff ? -1 : (int)items;
+  plan->grid = plan->work_items;  // upper bound; a launch uses min(its work items, 8 * (CUs / 8))
   plan->pairs_per_head = pairs;
 }
 
-void plan_for(const Request& r, int hp, int nw, IntraPlan* plan) {
-  switch (r.kind) {
-    case KIND_LLM_SCATTER: fill_plan<MapLlmScatter>(r, hp, nw, plan); break;
-    case KIND_LLM_GATHER1: fill_plan<MapLlmGather1>(r, hp, nw, plan); break;
-    case KIND_LLM_WINDOW: fill_plan<MapLlmWindow>(r, hp, nw, plan); break;
-    case KIND_IMG_SCATTER: fill_plan<MapImgScatter>(r, hp, nw, plan); break;
-    default: fill_plan<MapImgGather0>(r, hp, nw, plan); break;
-  }
-}
-
 // Host walk of the kernel's decomposition: sets -> row blocks -> wavefronts -> key tiles ->
-// 32-key blocks, with the same classification and per-element bound test as the device code.
+// 32-key blocks, with the same block tests and per-element bound test as the device code.
 template <class MAP>
 void model_walk(const IntraGeom& ge, int hp, int nw, uint8_t* count) {
   const int pos = nw * 32 / hp;
@@ -135,12 +194,12 @@ void model_walk(const IntraGeom& ge, int hp, int nw, uint8_t* count) {
   const int n_mblocks = (MAP::max_nq(ge) + pos - 1) / pos;
   for (int set = 0; set < n_sets; ++set) {
     MAP map(ge, set);
-    const int nq = map.nq(), nk = map.nk();
+    const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
     for (int mblk = 0; mblk < n_mblocks; ++mblk) {
       const int t0 = mblk * pos;
       if (t0 >= nq) continue;
       const int t1 = im_min(t0 + pos, nq) - 1;
-      const int kt_lo = map.klo(t0);
+      const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);
       const int kt_hi = im_min(map.khi(t1), nk - 1);
       const int ntiles = (kt_hi - kt_lo + intra::BN) / intra::BN;
       for (int pw = 0; pw < pos / 32; ++pw) {  // the wavefronts of one head
@@ -148,24 +207,22 @@ void model_walk(const IntraGeom& ge, int hp, int nw, uint8_t* count) {
         if (wq0 > t1) continue;
         const int wq_last = im_min(wq0 + 31, t1);
         const WaveBounds wb = wave_bounds(map, wq0, wq_last);
-        for (int tile = 0; tile < ntiles; ++tile) {
-          for (int b = 0; b < 2; ++b) {
-            const int sb_lo = kt_lo + tile * intra::BN + 32 * b;
-            const int cls = classify_block(wb, sb_lo);
-            if (cls == BLK_SKIP) continue;
-            for (int l = 0; l < 32; ++l) {
-              if (wq0 + l > t1) continue;  // rows the kernel computes but never stores
-              const int tq = wq0 + l;
-              const int lo = map.klo(tq), hi = im_min(map.khi(tq), nk - 1);
-              for (int e = 0; e < 32; ++e) {
-                const int key = sb_lo + e;
-                if (cls == BLK_PARTIAL && (key < lo || key > hi)) continue;
-                // a FULL block keeps every element: clamp the loaded row like the loader does
-                const int tk = im_min(key, nk - 1);
-                const int64_t qp = map.qpos(tq), kp = map.kpos(tk);
-                uint8_t& c8 = count[qp * S + kp];
-                if (c8 < 255) ++c8;
-              }
+        for (int blk = 0; blk < (intra::BN / 32) * ntiles; ++blk) {
+          const int sb_lo = kt_lo + 32 * blk;
+          if (!block_wanted(wb, kpre, sb_lo)) continue;
+          const bool unmasked = block_unmasked(wb, kpre, sb_lo);
+          for (int l = 0; l < 32; ++l) {
+            if (wq0 + l > t1) continue;  // rows the kernel computes but never stores
+            const int tq = wq0 + l;
+            const int lo = map.klo(tq), hi = im_min(map.khi(tq), nk - 1);
+            for (int e = 0; e < 32; ++e) {
+              const int key = sb_lo + e;
+              if (!unmasked && !key_visible(key, kpre, lo, hi)) continue;
+              // an unmasked block keeps every element: clamp the loaded row like the loader does
+              const int tk = im_min(key, nk - 1);
+              const int64_t qp = map.qpos(tq), kp = map.kpos(tk);
+              uint8_t& c8 = count[qp * S + kp];
+              if (c8 < 255) ++c8;
             }
           }
         }
@@ -173,6 +230,9 @@ void model_walk(const IntraGeom& ge, int hp, int nw, uint8_t* count) {
     }
   }
 }
+template <class MAP> struct ModelWalk {
+  static int go(const IntraGeom& ge, int hp, int nw, uint8_t* count) { model_walk<MAP>(ge, hp, nw, count); return 0; }
+};
 
 // One persistent workgroup per CU (LDS allows no more), in multiples of the 8 XCDs.
 int launch_grid(int work_items) {
@@ -198,13 +258,22 @@ int launch(const intra::KParams& p, int grid, hipStream_t stream) {
 }
 
 template <class MAP>
-int launch_hp8(const intra::KParams& p, int hp, int grid, hipStream_t stream) {
-  switch (hp) {
-    case 4: return launch<MAP, 4, 8>(p, grid, stream);
-    case 2: return launch<MAP, 2, 8>(p, grid, stream);
-    default: return launch<MAP, 1, 8>(p, grid, stream);
+struct LaunchMap {
+  static int go(const intra::KParams& p, int hp, int nw, int grid, hipStream_t stream) {
+    if (nw == 8) {
+      switch (hp) {
+        case 4: return launch<MAP, 4, 8>(p, grid, stream);
+        case 2: return launch<MAP, 2, 8>(p, grid, stream);
+        case 1: return launch<MAP, 1, 8>(p, grid, stream);
+      }
+    }
+    if (std::is_same<MAP, MapImgScatter>::value) {  // 64-query text chunks of gather0
+      if (hp == 2 && nw == 4) return launch<MapImgScatter, 2, 4>(p, grid, stream);
+      if (hp == 1 && nw == 2) return launch<MapImgScatter, 1, 2>(p, grid, stream);
+    }
+    return fail(INTRA_ERR_UNSUPPORTED, "no kernel for heads_per_block=%d, waves=%d", hp, nw);
   }
-}
+};
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -237,13 +306,8 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   if ((rc = check_strides("o", os, B, S, H))) return rc;
   if (!isfinite(scale)) return fail(INTRA_ERR_INVALID, "softmax_scale must be finite");
 
-  int hp, nw;
-  pick_shape(r.kind, H / Hkv, &hp, &nw);
-  IntraPlan plan;
-  plan_for(r, hp, nw, &plan);
-  if (plan.work_items <= 0) return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 work items");
-  const int grid = launch_grid(plan.work_items);
-  if (grid <= 0) return fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
+  if (ks[1] >= ((int64_t)1 << 31) || vs[1] >= ((int64_t)1 << 31))
+    return fail(INTRA_ERR_UNSUPPORTED, "k / v token stride must stay below 2^31 elements");
 
   intra::KParams p;
   p.q = static_cast<const uint16_t*>(q);
@@ -255,34 +319,36 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.v_bs = vs[0]; p.v_rs = vs[1]; p.v_hs = vs[2];
   p.o_bs = os[0]; p.o_rs = os[1]; p.o_hs = os[2];
   p.B = B; p.H = H; p.Hkv = Hkv; p.ratio = H / Hkv;
-  p.geom = r.geom;
   p.scale_log2 = fabsf(scale) * 1.4426950408889634f;
   if (p.scale_log2 < 1e-30f) p.scale_log2 = 1e-30f;  // scale 0: uniform weights without 0 * inf on masked scores
   p.negate_q = scale < 0.f;
-  if (ks[1] >= ((int64_t)1 << 31) || vs[1] >= ((int64_t)1 << 31))
-    return fail(INTRA_ERR_UNSUPPORTED, "k / v token stride must stay below 2^31 elements");
   p.k_rs_bytes = (uint32_t)(ks[1] * 2);
   p.v_rs_bytes = (uint32_t)(vs[1] * 2);
-  p.n_sets = plan.n_sets;
-  p.n_mblocks = plan.n_mblocks;
-  p.hgroups = p.ratio / hp;
-  p.n_pairs = B * Hkv * plan.n_sets;
-  p.items_per_pair = p.hgroups * plan.n_mblocks;
-  p.n_slots = plan.work_items / 8;
 
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  switch (r.kind) {
-    case KIND_LLM_SCATTER: return launch_hp8<MapLlmScatter>(p, hp, grid, st);
-    case KIND_LLM_GATHER1: return launch_hp8<MapLlmGather1>(p, hp, grid, st);
-    case KIND_LLM_WINDOW: return launch_hp8<MapLlmWindow>(p, hp, grid, st);
-    case KIND_IMG_SCATTER: return launch_hp8<MapImgScatter>(p, hp, grid, st);
-    default:
-      switch (hp) {
-        case 4: return launch<MapImgGather0, 4, 8>(p, grid, st);
-        case 2: return launch<MapImgGather0, 2, 4>(p, grid, st);
-        default: return launch<MapImgGather0, 1, 2>(p, grid, st);
-      }
+  Phase ph[2];
+  const int n_phases = phases_for(r, default_hp(H / Hkv), ph);
+  PhaseDims dims[2];
+  for (int i = 0; i < n_phases; ++i) {
+    dims[i] = by_map<DimsOf>(ph[i].map, r, ph[i]);
+    if (dims[i].work_items <= 0 || dims[i].n_pairs <= 0)
+      return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 work items");
   }
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  for (int i = 0; i < n_phases; ++i) {  // the launches write disjoint rows of o
+    const int grid = launch_grid(dims[i].work_items);
+    if (grid <= 0)
+      return fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
+    p.geom = ph[i].geom;
+    p.n_sets = dims[i].n_sets;
+    p.n_mblocks = dims[i].n_mblocks;
+    p.hgroups = dims[i].hgroups;
+    p.n_pairs = dims[i].n_pairs;
+    p.items_per_pair = dims[i].hgroups * dims[i].n_mblocks;
+    p.n_slots = dims[i].work_items / 8;
+    rc = by_map<LaunchMap>(ph[i].map, p, ph[i].hp, ph[i].nw, grid, st);
+    if (rc) return rc;
+  }
+  return INTRA_OK;
 }
 
 }  // namespace
@@ -316,9 +382,7 @@ int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, 
   Request r;
   int rc = make_request(domain, pattern, B, S, H, Hkv, arg0, arg1, &r);
   if (rc) return rc;
-  int hp, nw;
-  pick_shape(r.kind, H / Hkv, &hp, &nw);
-  plan_for(r, hp, nw, plan);
+  plan_for(r, default_hp(H / Hkv), plan);
   return INTRA_OK;
 }
 
@@ -329,19 +393,12 @@ int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int hea
   Request r;
   int rc = make_request(domain, pattern, 1, S, 1, 1, arg0, arg1, &r);
   if (rc) return rc;
-  int hp, nw;
-  pick_shape(r.kind, 1, &hp, &nw);
-  if (heads_per_block > 0) hp = heads_per_block;
-  if (waves > 0) nw = waves;
-  if (!shape_ok(r.kind, hp, nw))
-    return fail(INTRA_ERR_INVALID, "no kernel for heads_per_block=%d, waves=%d", hp, nw);
-  switch (r.kind) {
-    case KIND_LLM_SCATTER: model_walk<MapLlmScatter>(r.geom, hp, nw, count); break;
-    case KIND_LLM_GATHER1: model_walk<MapLlmGather1>(r.geom, hp, nw, count); break;
-    case KIND_LLM_WINDOW: model_walk<MapLlmWindow>(r.geom, hp, nw, count); break;
-    case KIND_IMG_SCATTER: model_walk<MapImgScatter>(r.geom, hp, nw, count); break;
-    default: model_walk<MapImgGather0>(r.geom, hp, nw, count); break;
-  }
+  const int hp = heads_per_block > 0 ? heads_per_block : 1;
+  if ((hp != 1 && hp != 2 && hp != 4) || (waves > 0 && waves != 8))
+    return fail(INTRA_ERR_INVALID, "no kernel for heads_per_block=%d, waves=%d", hp, waves);
+  Phase ph[2];
+  const int n_phases = phases_for(r, hp, ph);
+  for (int i = 0; i < n_phases; ++i) by_map<ModelWalk>(ph[i].map, ph[i].geom, ph[i].hp, ph[i].nw, count);
   return INTRA_OK;
 }
 

@@ -161,7 +161,8 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   const int t0 = mblk * POS;
   if (t0 >= nq) continue;
   const int t1 = im_min(t0 + POS, nq) - 1;
-  const int kt_lo = map.klo(t0);
+  const int kpre = map.kpre();                            // keys every query of the set sees (0 if none)
+  const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);  // first key the row block looks at
   const int kt_hi = im_min(map.khi(t1), nk - 1);
   const int ntiles = (kt_hi - kt_lo + BN) / BN;
 
@@ -175,16 +176,20 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   const int lo_l = map.klo(tq);
   const int hi_l = im_min(map.khi(tq), nk - 1);
   WaveBounds wb = wave_bounds(map, im_min(wq0, t1), wq_last);
-  // 32-key blocks (counted from kt_lo) this wavefront has to look at; blocks inside
-  // [f_lo, f_hi] need no mask
+  // 32-key blocks (counted from kt_lo) this wavefront has to look at: those of its own key range
+  // and, for maps with a prefix, the prefix blocks in front of it.
   int bw_lo = __builtin_amdgcn_readfirstlane((wb.w_lo - kt_lo) / 32);
   int bw_hi = __builtin_amdgcn_readfirstlane((wb.w_hi - kt_lo) / 32);
+  int bp_hi = MAP::kHasPrefix ? (kpre - 1) / 32 : -1;  // last prefix block
   if (!wave_active) {
     bw_lo = 1;
     bw_hi = 0;
+    bp_hi = -1;
   }
-  const int f_lo = __builtin_amdgcn_readfirstlane(wb.f_lo);
-  const int f_hi = __builtin_amdgcn_readfirstlane(wb.f_hi);
+  wb.f_lo = __builtin_amdgcn_readfirstlane(wb.f_lo);
+  wb.f_hi = __builtin_amdgcn_readfirstlane(wb.f_hi);
+  wb.w_lo = __builtin_amdgcn_readfirstlane(wb.w_lo);
+  wb.w_hi = __builtin_amdgcn_readfirstlane(wb.w_hi);
 
   const int hq = kvh * p.ratio + hg * HP + hw;
   const int64_t qpos = map.qpos(tq);
@@ -287,7 +292,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       int key = kb32 + 8 * (e >> 2) + 4 * h32 + (e & 3);
-      if (key < lo_l || key > hi_l) s[e] = -INFINITY;
+      if (!key_visible(key, kpre, lo_l, hi_l)) s[e] = -INFINITY;
     }
   };
   auto block_max = [&](const floatx16& s) {
@@ -383,23 +388,33 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 
   // Step j: softmax + PV of key block j (scores in `cur`, V rows at voff) and QK^T of key block
   // j+1 into `nxt` (its K rows at koff; those of block j+2 at koff_next).  A wavefront runs the
-  // steps jq..jp with jq = bw_lo - 1: in step jq only the QK^T half matters, so its scores are
-  // preset to -inf (weights 0); in step jp the QK^T half computes a block nobody reads (masked
-  // to -inf so that it cannot move the reference).  That keeps one code path through the
-  // accumulators.  Blocks not inside [f_lo, f_hi] get the per-element mask.
-  const int jq = bw_lo - 1, jp = bw_hi;
-  auto needs_mask = [&](int j) {
-    const int kb32 = kt_lo + 32 * j;
-    return j >= jp + 1 || kb32 < f_lo || kb32 + 31 > f_hi;
-  };
+  // steps jq..jp for a run of blocks jq+1..jp it looks at: in step jq only the QK^T half matters,
+  // so its scores are preset to -inf (weights 0); in step jp the QK^T half computes a block the
+  // wavefront does not look at, which the per-element mask turns into -inf.  That keeps one code
+  // path through the accumulators.  Maps with a prefix have two such runs (prefix blocks, own
+  // range); they are merged when they touch.
+  int jq1 = bw_lo - 1, jp1 = bw_hi, jq2 = 1, jp2 = 0;
+  if (MAP::kHasPrefix && bp_hi >= 0) {
+    if (bw_lo - 1 <= bp_hi) {  // the ranges touch: one run from the first prefix block on
+      jq1 = -1;
+      jp1 = im_max(bw_hi, bp_hi);
+    } else {
+      jq1 = -1;
+      jp1 = bp_hi;
+      jq2 = bw_lo - 1;
+      jp2 = bw_hi;
+    }
+  }
+  auto needs_mask = [&](int j) { return !block_unmasked(wb, kpre, kt_lo + 32 * j); };
   auto step = [&](int j, floatx16& cur, floatx16& nxt, int koff, int koff_next, int voff, auto with_loader,
                   int i, int kdst, int vdst) {
     if (decltype(with_loader)::value) {
       load_k(i + 3, kdst);
       load_v(i + 2, vdst);
     }
-    if (j < jq || j > jp) return;
-    if (j == jq) {
+    const bool in1 = j >= jq1 && j <= jp1, in2 = j >= jq2 && j <= jp2;
+    if (!in1 && !in2) return;
+    if (j == jq1 || (in2 && j == jq2)) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) cur[e] = -INFINITY;
 #pragma unroll
@@ -429,7 +444,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   }
   scale_q();
   tile_barrier<PER_TILE>();
-  if (jq < 0 && jp >= 0) {
+  if (jq1 < 0 && jp1 >= 0) {
     qk_block(s0, 0);
     settle(s0, block_max(s0), needs_mask(0), kt_lo);
 #pragma unroll

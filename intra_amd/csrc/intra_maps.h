@@ -39,6 +39,8 @@ struct IntraGeom {
   int window;    // LLM window width in keys (>= 64)
   int width;     // image latent grid side (tokens)
   int text_len;  // image: text tokens in front of the grid
+  int text_only; // image scatter: only the text queries of each group (the text rows of gather0)
+  int pg;        // image gather0: 8x8 patches per set (a run of pg patches in one patch row)
 };
 
 IM_HD int im_min(int a, int b) { return a < b ? a : b; }
@@ -46,6 +48,8 @@ IM_HD int im_max(int a, int b) { return a > b ? a : b; }
 
 // ---------------------------------------------------------------- LLM scatter: token i in group i % G
 struct MapLlmScatter {
+  static constexpr bool kHasPrefix = false;
+  IM_HD int kpre() const { return 0; }
   int G, g, n;
   static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
   static IM_HD int max_nq(const IntraGeom& ge) { return (ge.S + ge.G - 1) / ge.G; }
@@ -66,6 +70,8 @@ struct MapLlmScatter {
 // Token p = (G*G)*a + G*g + r (r < G) is in-set index G*a + r of group g; positions grow with the
 // in-set index, so causality in positions equals causality in in-set indices.
 struct MapLlmGather1 {
+  static constexpr bool kHasPrefix = false;
+  IM_HD int kpre() const { return 0; }
   int G, g, n;
   static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
   static IM_HD int max_nq(const IntraGeom& ge) {
@@ -89,6 +95,8 @@ struct MapLlmGather1 {
 
 // -------------------------- LLM window: 64-query blocks see themselves plus window-64 earlier tokens
 struct MapLlmWindow {
+  static constexpr bool kHasPrefix = false;
+  IM_HD int kpre() const { return 0; }
   int S, lookback;
   static IM_HD int num_sets(const IntraGeom&) { return 1; }
   static IM_HD int max_nq(const IntraGeom& ge) { return ge.S; }
@@ -107,9 +115,13 @@ struct MapLlmWindow {
 // ------------- image scatter: 8 groups, grid token (r, c) in group (r%2)*4 + c%4, text chunk j rides
 // with group j; every query sees all text keys plus the grid keys of its own group.
 struct MapImgScatter {
-  int W, T, chunk, j, a, b, wq, nimg;
+  static constexpr bool kHasPrefix = false;
+  IM_HD int kpre() const { return 0; }
+  int W, T, chunk, j, a, b, wq, nimg, text_only;
   static IM_HD int num_sets(const IntraGeom&) { return 8; }
-  static IM_HD int max_nq(const IntraGeom& ge) { return ge.text_len / 8 + ge.width * ge.width / 8; }
+  static IM_HD int max_nq(const IntraGeom& ge) {
+    return ge.text_only ? ge.text_len / 8 : ge.text_len / 8 + ge.width * ge.width / 8;
+  }
   IM_HD MapImgScatter(const IntraGeom& ge, int set) {
     W = ge.width;
     T = ge.text_len;
@@ -119,9 +131,10 @@ struct MapImgScatter {
     b = set & 3;
     wq = W / 4;
     nimg = W * W / 8;
+    text_only = ge.text_only;
   }
   IM_HD int imgpos(int u) const { return T + (a + 2 * (u / wq)) * W + b + 4 * (u % wq); }
-  IM_HD int nq() const { return chunk + nimg; }
+  IM_HD int nq() const { return text_only ? chunk : chunk + nimg; }
   IM_HD int nk() const { return T + nimg; }
   IM_HD int qpos(int t) const { return t < chunk ? chunk * j + t : imgpos(t - chunk); }
   IM_HD int kpos(int t) const { return t < T ? t : imgpos(t - T); }
@@ -129,49 +142,54 @@ struct MapImgScatter {
   IM_HD int khi(int) const { return T + nimg - 1; }
 };
 
-// ---- image gather0: every 8x8 patch of grid queries sees all text plus a 16x16 grid window around
-// it (shifted inwards at the borders); text queries keep their scatter rows.  Sets 0..7 are the text
-// chunks (keys = scatter key list of group j), sets 8.. are the patches in row-major patch order.
-struct MapImgGather0 {
-  int W, T, chunk, m, r0, c0, qr, qc;
-  MapImgScatter sc;
-  static IM_HD int num_sets(const IntraGeom& ge) { return 8 + (ge.width / 8) * (ge.width / 8); }
-  static IM_HD int max_nq(const IntraGeom& ge) { return im_max(ge.text_len / 8, 64); }
+// ---- image gather0, grid queries: every 8x8 patch of grid queries sees all text plus a 16x16 grid
+// window around it (shifted inwards at the borders).  A set is a run of pg patches of one patch
+// row, so that the text keys (a prefix every query sees) and most of the window keys are shared.
+// The window keys of the set are the union of the patches' windows, cut into blocks of 4 grid
+// columns x 16 grid rows = 64 keys; window starts are multiples of 4, so a patch sees exactly 4
+// consecutive blocks.  The text queries of gather0 keep their scatter rows and are computed with
+// MapImgScatter in text_only mode.
+struct MapImgPatch {
+  static constexpr bool kHasPrefix = true;
+  int W, T, pg, np, R, C0, r0, cfirst, nblk;
   static IM_HD int win_start(int idx, int np) {
     if (idx == np - 1) return idx * 8 - 8;
     if (idx == 0) return 0;
     return idx * 8 - 4;
   }
-  IM_HD MapImgGather0(const IntraGeom& ge, int set) : sc(ge, set < 8 ? set : 0) {
+  static IM_HD int num_sets(const IntraGeom& ge) { return (ge.width / 8) * ((ge.width / 8) / ge.pg); }
+  static IM_HD int max_nq(const IntraGeom& ge) { return 64 * ge.pg; }
+  IM_HD MapImgPatch(const IntraGeom& ge, int set) {
     W = ge.width;
     T = ge.text_len;
-    chunk = T / 8;
-    m = set;
-    int np = W / 8;
-    int P = set < 8 ? 0 : set - 8;
-    int R = P / np, C = P % np;
-    qr = 8 * R;
-    qc = 8 * C;
+    pg = ge.pg;
+    np = W / 8;
+    const int per_row = np / pg;
+    R = set / per_row;
+    C0 = (set % per_row) * pg;
     r0 = win_start(R, np);
-    c0 = win_start(C, np);
+    cfirst = win_start(C0, np);
+    nblk = (win_start(C0 + pg - 1, np) + 16 - cfirst) / 4;
   }
-  IM_HD int nq() const { return m < 8 ? chunk : 64; }
-  IM_HD int nk() const { return m < 8 ? sc.nk() : T + 256; }
-  IM_HD int qpos(int t) const { return m < 8 ? chunk * m + t : T + (qr + (t >> 3)) * W + qc + (t & 7); }
+  IM_HD int nq() const { return 64 * pg; }
+  IM_HD int nk() const { return T + 64 * nblk; }
+  IM_HD int kpre() const { return T; }
+  IM_HD int qpos(int t) const {
+    const int w = t & 63;
+    return T + (8 * R + (w >> 3)) * W + 8 * (C0 + (t >> 6)) + (w & 7);
+  }
   IM_HD int kpos(int t) const {
-    if (m < 8) return sc.kpos(t);
     if (t < T) return t;
-    int u = t - T;
-    return T + (r0 + (u >> 4)) * W + c0 + (u & 15);
+    const int u = t - T;
+    return T + (r0 + ((u >> 2) & 15)) * W + cfirst + 4 * (u >> 6) + (u & 3);
   }
-  IM_HD int klo(int) const { return 0; }
-  IM_HD int khi(int) const { return nk() - 1; }
+  IM_HD int klo(int tq) const { return T + 16 * (win_start(C0 + (tq >> 6), np) - cfirst); }
+  IM_HD int khi(int tq) const { return klo(tq) + 255; }
 };
 
-// --------------------------------------------------------------------------- tile classification
-// A wavefront owns the queries wq0..wq_last of a set and looks at the 32 keys sb_lo..sb_lo+31.
-enum : int { BLK_SKIP = 0, BLK_FULL = 1, BLK_PARTIAL = 2 };
-
+// --------------------------------------------------------------------------- block classification
+// A wavefront owns the queries wq0..wq_last of a set.  Query tq sees the keys below kpre() (the
+// prefix, if the map has one) and klo(tq)..min(khi(tq), nk-1).
 struct WaveBounds {
   int w_lo, w_hi;  // union of the key ranges of the wavefront's queries
   int f_lo, f_hi;  // intersection of them
@@ -188,9 +206,11 @@ IM_HD WaveBounds wave_bounds(const MAP& map, int wq0, int wq_last) {
   return wb;
 }
 
-IM_HD int classify_block(const WaveBounds& wb, int sb_lo) {
-  int sb_hi = sb_lo + 31;
-  if (sb_lo > wb.w_hi || sb_hi < wb.w_lo) return BLK_SKIP;
-  if (sb_lo >= wb.f_lo && sb_hi <= wb.f_hi) return BLK_FULL;
-  return BLK_PARTIAL;
+// Does the wavefront look at the 32 keys sb_lo..sb_lo+31 at all, and can it skip the mask?
+IM_HD bool block_wanted(const WaveBounds& wb, int kpre, int sb_lo) {
+  return sb_lo < kpre || (sb_lo <= wb.w_hi && sb_lo + 31 >= wb.w_lo);
 }
+IM_HD bool block_unmasked(const WaveBounds& wb, int kpre, int sb_lo) {
+  return sb_lo + 31 < kpre || (sb_lo >= kpre && sb_lo >= wb.f_lo && sb_lo + 31 <= wb.f_hi);
+}
+IM_HD bool key_visible(int key, int kpre, int lo, int hi) { return key < kpre || (key >= lo && key <= hi); }

@@ -38,6 +38,20 @@ def test_plan_headline(lib):
     assert p.pairs_per_head == 67125248 and 0 < p.lds_bytes <= 160 * 1024
 
 
+def test_plan_gather0_is_two_launches(lib):
+    # grid rows: sets of 4 / 2 / 1 neighbouring 8x8 patches; text rows: 8 text-only scatter sets
+    for H, Hkv, hp, pg in ((24, 24, 1, 4), (16, 8, 2, 2), (32, 8, 4, 1)):
+        rc, p = _plan(lib, 1, 4, 1, 16896, H, Hkv, 128, 512)
+        assert rc == 0 and p.launches == 2
+        assert (p.heads_per_block, p.waves, p.pos_per_block) == (hp, 8, 256 // hp)
+        assert (p.n_sets, p.n_mblocks) == (16 * 16 // pg, 1)
+        patch_items = 8 * -(-Hkv * p.n_sets // 8) * (H // Hkv // hp)
+        text_items = 8 * -(-Hkv * 8 // 8) * (H // Hkv // hp)
+        assert p.work_items == patch_items + text_items
+    rc, p = _plan(lib, 1, 0, 1, 16896, 24, 24, 128, 512)
+    assert rc == 0 and p.launches == 1
+
+
 @pytest.mark.parametrize("domain,pattern,kind,S,a0,a1", [
     (0, 0, "llm/scatter", 1000, 3, 576), (0, 1, "llm/gather1", 3000, 8, 576),
     (0, 4, "llm/window", 3000, 8, 1000), (1, 0, "image/scatter", 4608, 64, 512),
@@ -120,8 +134,7 @@ IMG_CASES = [(16, 64), (24, 16), (32, 512), (64, 512), (40, 8)]
 @pytest.mark.parametrize("hp", [1, 2, 4])
 def test_kernel_decomposition_equals_mask_image(lib, W, T, kind, pattern, hp):
     S = T + W * W
-    nw = 2 * hp if pattern == 4 else 8
-    count = _model(lib, 1, pattern, S, W, T, hp, nw)
+    count = _model(lib, 1, pattern, S, W, T, hp, 8)
     want = oracle.mask_rows(kind, S, width=W, text_len=T)
     assert count.max() <= 1
     assert torch.equal(count.bool(), want)
