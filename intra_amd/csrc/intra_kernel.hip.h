@@ -79,7 +79,7 @@ constexpr int GROUP_STRIDE = 1024 + 16;
 constexpr int TILE_BYTES = (BN / 4) * GROUP_STRIDE;
 constexpr int KTILE = TILE_BYTES;
 constexpr int VTILE = TILE_BYTES;
-constexpr int NKBUF = 4, NVBUF = 3;   // K tiles i-1 (being overwritten) .. i+2, V tiles i-1 .. i+1
+constexpr int NKBUF = 4, NVBUF = 4;   // tiles i-1 (being overwritten) .. i+2 of K and of V
 constexpr int VBASE = NKBUF * KTILE;  // K ring then V ring
 constexpr int LDS_BYTES = NKBUF * KTILE + NVBUF * VTILE;
 constexpr int BLOCK32 = 8 * GROUP_STRIDE;  // 32 rows
@@ -140,31 +140,143 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   const int xcd = blockIdx.x & 7;
   const int wgs_per_xcd = gridDim.x >> 3;
   const int wg_in_xcd = blockIdx.x >> 3;
-  for (int round = 0;; ++round) {
-  const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
-  if (slot >= p.n_slots) break;
-  if (round > 0) tile_barrier<0>();  // everybody is done with the LDS tiles of the previous item
-  const int pair = (slot / p.items_per_pair) * 8 + xcd;
-  if (pair >= p.n_pairs) continue;
-  const int rem = slot % p.items_per_pair;
-  const int mblk = p.n_mblocks - 1 - rem / p.hgroups;
-  const int hg = rem % p.hgroups;
-  const int nbh = p.B * p.Hkv;
-  const int set = pair / nbh;
-  const int bh = pair % nbh;
-  const int batch = bh / p.Hkv;
-  const int kvh = bh % p.Hkv;
+  struct Where {
+    int round, set, batch, kvh, mblk, hg;
+  };
+  // first non-empty work item of this workgroup at or after `round`
+  auto locate = [&](int round, Where& w) {
+    for (;; ++round) {
+      const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
+      if (slot >= p.n_slots) return false;
+      const int pair = (slot / p.items_per_pair) * 8 + xcd;
+      if (pair >= p.n_pairs) continue;
+      const int rem = slot % p.items_per_pair;
+      const int nbh = p.B * p.Hkv;
+      const int bh = pair % nbh;
+      w.round = round;
+      w.set = pair / nbh;
+      w.batch = bh / p.Hkv;
+      w.kvh = bh % p.Hkv;
+      w.mblk = p.n_mblocks - 1 - rem / p.hgroups;
+      w.hg = rem % p.hgroups;
+      if (w.mblk * POS >= MAP(p.geom, w.set).nq()) continue;
+      return true;
+    }
+  };
+  // Key range of a row block: tiles of BN keys counted from kt_lo.
+  struct Range {
+    int kt_lo, ntiles;
+  };
+  auto range_of = [&](const MAP& map, int mblk) {
+    const int t0 = mblk * POS;
+    const int t1 = im_min(t0 + POS, map.nq()) - 1;
+    const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);  // first key the row block looks at
+    const int kt_hi = im_min(map.khi(t1), map.nk() - 1);
+    return Range{kt_lo, (kt_hi - kt_lo + BN) / BN};
+  };
 
+  // ---------------------------------------------------------------- loader: HBM rows -> LDS
+  // One global_load_lds_dwordx4 moves a 4-row group: lane L fetches 16 bytes of row L/16 and the
+  // hardware writes the 64 x 16 bytes to consecutive LDS addresses from M0, so lane L has to
+  // fetch the chunk that belongs into slot L%16 of its row.  No VGPR staging and no LDS store
+  // instructions; rows past the last key are clamped to it.
+  //
+  // The K/V tiles of all work items of this workgroup form one stream that runs through the LDS
+  // ring without a break: the loader has its own cursor (`fd`), three tiles ahead of the
+  // computation, and moves on to the next work item when it has requested the last tile of one.
+  // So the first tiles of a work item arrive while the previous one is still computing.
+  constexpr int GROUPS_PER_WAVE = (BN / 4) / NW;
+  static_assert((BN / 4) % NW == 0, "tile groups must split evenly over the wavefronts");
+  const int ld_row = lane >> 4;                                  // row of the group this lane fetches
+  const uint32_t ld_col = (((lane & 15) ^ (4 * ld_row)) << 4);   // byte column it fetches
+  const uint32_t k_rs_b = p.k_rs_bytes, v_rs_b = p.v_rs_bytes;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  struct Feed {
+    MAP map;
+    Range rg;
+    int nk, tile, round;
+    bool more;
+    const char *kbase, *vbase;
+  };
+  auto feed_for = [&](const Where& w) {
+    const MAP map(p.geom, w.set);
+    return Feed{map, range_of(map, w.mblk), map.nk(), 0, w.round, true,
+                reinterpret_cast<const char*>(p.k + w.batch * p.k_bs + w.kvh * p.k_hs),
+                reinterpret_cast<const char*>(p.v + w.batch * p.v_bs + w.kvh * p.v_hs)};
+  };
+  Where cw;
+  if (!locate(0, cw)) return;
+  Feed fd = feed_for(cw);
+  auto feed_tile = [&](int slot_off) {  // request the next K and V tile of the stream into a ring slot
+#pragma unroll
+    for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
+      const int grp = wave * GROUPS_PER_WAVE + gi;
+      const int tk = im_min(fd.rg.kt_lo + fd.tile * BN + 4 * grp + ld_row, fd.nk - 1);
+      const uint32_t pos = fd.map.kpos(tk);
+      dma_group(fd.kbase + ((uint64_t)pos * k_rs_b + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
+      dma_group(fd.vbase + ((uint64_t)pos * v_rs_b + ld_col), lds_base + VBASE + slot_off + grp * GROUP_STRIDE);
+    }
+    ++fd.tile;
+    if (fd.tile == fd.rg.ntiles && fd.more) {
+      Where w;
+      if (locate(fd.round + 1, w)) fd = feed_for(w);
+      else fd.more = false;  // nothing left: keep requesting the (clamped) last row, nobody reads it
+    }
+  };
+  constexpr int PER_TILE = 2 * GROUPS_PER_WAVE;  // requests per wavefront per tile (K + V)
+
+  // K operand (A of S^T = K Q^T): lane reads 16 bytes of key row l32 at head dims 16*ks + 8*h32
+  int kaddr[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks)
+    kaddr[ks] = (l32 >> 2) * GROUP_STRIDE + (l32 & 3) * 256 + (((2 * ks + h32) ^ (4 * (l32 & 3))) << 4);
+  // V^T operand (A of O^T = V^T P^T) through transposing reads.  Within each group of 16 lanes,
+  // lane i supplies the address of 4 head dims (4*(i%4)..) of key row i/4 and receives head dim i
+  // of those 4 key rows.  Lane groups 0/1 take head dims 0-15/16-31 of a 32-dim block, the upper
+  // 32 lanes the key rows 4..7 of each 8 (the next 4-row group).  vaddr[db]: 32-dim block db.
+  int vaddr[4];
+  {
+    const int i16 = lane & 15, g2 = (lane >> 4) & 1, ri = i16 >> 2;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+      vaddr[db] = VBASE + h32 * GROUP_STRIDE + ri * 256 + (((4 * db + 2 * g2 + ((i16 & 3) >> 1)) ^ (4 * ri)) << 4) +
+                  8 * (i16 & 1);
+  }
+  // Q^T fragments: lane holds query l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
+  bf16x8 qf[8];
+  // this lane's query row of a work item (clamped to the last row of the row block)
+  auto q_row = [&](const Where& w) {
+    const MAP map(p.geom, w.set);
+    const int t1 = im_min(w.mblk * POS + POS, map.nq()) - 1;
+    const int tq = im_min(w.mblk * POS + (wave / HP) * 32 + l32, t1);
+    const int hq = w.kvh * p.ratio + w.hg * HP + wave % HP;
+    return w.batch * p.q_bs + (int64_t)map.qpos(tq) * p.q_rs + hq * p.q_hs + h32 * 8;
+  };
+  auto load_q = [&](const Where& w) {
+    const uint16_t* qrow = p.q + q_row(w);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + ks * 16);
+  };
+
+  // Ring slots (byte offsets into the K ring; the V ring uses the same offsets behind VBASE) of
+  // the stream tiles i, i+1, i+2, i+3 seen from the computation; they rotate once per tile and
+  // carry on from one work item to the next.
+  int k0 = 0, k1 = KTILE, k2 = 2 * KTILE, k3 = 3 * KTILE;
+  feed_tile(k0);
+  feed_tile(k1);
+  feed_tile(k2);
+  load_q(cw);  // after the tile requests: the load counter is in order, so Q arrives last
+
+  for (;;) {
+  const int set = cw.set, batch = cw.batch, kvh = cw.kvh, mblk = cw.mblk, hg = cw.hg;
   const MAP map(p.geom, set);
   const int nq = map.nq();
   const int nk = map.nk();
   const int t0 = mblk * POS;
-  if (t0 >= nq) continue;
   const int t1 = im_min(t0 + POS, nq) - 1;
-  const int kpre = map.kpre();                            // keys every query of the set sees (0 if none)
-  const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);  // first key the row block looks at
-  const int kt_hi = im_min(map.khi(t1), nk - 1);
-  const int ntiles = (kt_hi - kt_lo + BN) / BN;
+  const int kpre = map.kpre();  // keys every query of the set sees (0 if none)
+  const Range rg = range_of(map, mblk);
+  const int kt_lo = rg.kt_lo, ntiles = rg.ntiles;
 
   // ---------------------------------------------------------------- this wavefront's queries
   const int hw = wave % HP;
@@ -193,58 +305,10 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 
   const int hq = kvh * p.ratio + hg * HP + hw;
   const int64_t qpos = map.qpos(tq);
-
-  // Q^T fragments: lane holds query l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
-  bf16x8 qf[8];
-  auto scale_q = [&] {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
-    if (p.negate_q) {
+  if (p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
-        qf[ks] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, qf[ks]) ^ 0x80008000u);
-    }
-  };
-
-  // ---------------------------------------------------------------- loader: HBM rows -> LDS
-  // One global_load_lds_dwordx4 moves a 4-row group: lane L fetches 16 bytes of row L/16 and the
-  // hardware writes the 64 x 16 bytes to consecutive LDS addresses from M0, so lane L has to
-  // fetch the chunk that belongs into slot L%16 of its row.  No VGPR staging and no LDS store
-  // instructions; rows past the last key are clamped to it.
-  constexpr int GROUPS_PER_WAVE = (BN / 4) / NW;
-  static_assert((BN / 4) % NW == 0, "tile groups must split evenly over the wavefronts");
-  const char* kbase = reinterpret_cast<const char*>(p.k + batch * p.k_bs + kvh * p.k_hs);
-  const char* vbase = reinterpret_cast<const char*>(p.v + batch * p.v_bs + kvh * p.v_hs);
-  const int ld_row = lane >> 4;                                  // row of the group this lane fetches
-  const uint32_t ld_col = (((lane & 15) ^ (4 * ld_row)) << 4);   // byte column it fetches
-  const uint32_t k_rs_b = p.k_rs_bytes, v_rs_b = p.v_rs_bytes;
-  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
-  auto load_tile = [&](const char* base, uint32_t rs_b, int tile, int lds_off) {
-#pragma unroll
-    for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
-      const int grp = wave * GROUPS_PER_WAVE + gi;
-      const int tk = im_min(kt_lo + tile * BN + 4 * grp + ld_row, nk - 1);
-      const uint32_t pos = map.kpos(tk);
-      dma_group(base + ((uint64_t)pos * rs_b + ld_col), lds_base + lds_off + grp * GROUP_STRIDE);  // one 32x32+64 mad
-    }
-  };
-  auto load_k = [&](int tile, int kbuf_off) { load_tile(kbase, k_rs_b, tile, kbuf_off); };
-  auto load_v = [&](int tile, int vbuf_off) { load_tile(vbase, v_rs_b, tile, VBASE + vbuf_off); };
-
-  // K operand (A of S^T = K Q^T): lane reads 16 bytes of key row l32 at head dims 16*ks + 8*h32
-  int kaddr[8];
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks)
-    kaddr[ks] = (l32 >> 2) * GROUP_STRIDE + (l32 & 3) * 256 + (((2 * ks + h32) ^ (4 * (l32 & 3))) << 4);
-  // V^T operand (A of O^T = V^T P^T) through transposing reads.  Within each group of 16 lanes,
-  // lane i supplies the address of 4 head dims (4*(i%4)..) of key row i/4 and receives head dim i
-  // of those 4 key rows.  Lane groups 0/1 take head dims 0-15/16-31 of a 32-dim block, the upper
-  // 32 lanes the key rows 4..7 of each 8 (the next 4-row group).  vaddr[db]: 32-dim block db.
-  int vaddr[4];
-  {
-    const int i16 = lane & 15, g2 = (lane >> 4) & 1, ri = i16 >> 2;
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-      vaddr[db] = VBASE + h32 * GROUP_STRIDE + ri * 256 + (((4 * db + 2 * g2 + ((i16 & 3) >> 1)) ^ (4 * ri)) << 4) +
-                  8 * (i16 & 1);
+    for (int ks = 0; ks < 8; ++ks)
+      qf[ks] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, qf[ks]) ^ 0x80008000u);
   }
 
   // ---------------------------------------------------------------- running softmax state
@@ -260,7 +324,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   // for every query whose scores stay within +-60 of it; it is re-centred on a block's maximum
   // when that maximum leaves this band upwards, or downwards before anything was accumulated.
   float mref = 0.f;
-  float l_run = 0.f;
+  float l_acc[2] = {0.f, 0.f};  // two partial row sums of the weights (summed at the end)
   const float c = p.scale_log2;  // |softmax_scale| * log2(e)
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
@@ -312,12 +376,15 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
       mx = block_max(nxt);
     }
     const float mxs = __builtin_fmaf(mx, c, -mref);  // block maximum in exponent units
+    if (__builtin_amdgcn_ballot_w64(__builtin_fabsf(mxs) > 60.f) == 0) return;  // the usual case
+    const float l_run = l_acc[0] + l_acc[1];
     const bool need = mxs > 60.f || (l_run == 0.f && mxs < -60.f && mxs > -INFINITY);
     if (__builtin_amdgcn_ballot_w64(need) != 0) {
       const float delta = need ? mxs : 0.f;
       const float alpha = l_run == 0.f ? 1.f : __builtin_amdgcn_exp2f(-delta);
       mref += delta;
-      l_run *= alpha;
+      l_acc[0] *= alpha;
+      l_acc[1] *= alpha;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -337,7 +404,6 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   bf16x8 ka[8];
   auto steady = [&](const floatx16& s, floatx16& n, int koff_next, int voff, bool mask_next, int kb32_next) {
     bf16x8 va[8], pb[2];
-    float rs[2] = {0.f, 0.f};
     float px[8][2];
     auto stage_e = [&](int u) {
       px[u][0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u], c, -mref));
@@ -346,7 +412,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     auto stage_c = [&](int u) {
       floatx2 f = {px[u][0], px[u][1]};
       bf16x2 h = __builtin_convertvector(f, bf16x2);
-      rs[u & 1] = __builtin_amdgcn_fdot2_f32_bf16(h, ones2, rs[u & 1], false);  // sums what PV multiplies
+      l_acc[u & 1] = __builtin_amdgcn_fdot2_f32_bf16(h, ones2, l_acc[u & 1], false);  // sums what PV multiplies
       pb[u >> 2][2 * (u & 3)] = h[0];
       pb[u >> 2][2 * (u & 3) + 1] = h[1];
     };
@@ -382,7 +448,6 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
       if (j == 7) m1 = fmaxf(fmaxf(m1, n[12]), fmaxf(n[13], fmaxf(n[14], n[15])));
       __builtin_amdgcn_sched_barrier(0);
     }
-    l_run += rs[0] + rs[1];
     settle(n, lane_xor32_max(fmaxf(m0, m1)), mask_next, kb32_next);
   };
 
@@ -407,11 +472,8 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   }
   auto needs_mask = [&](int j) { return !block_unmasked(wb, kpre, kt_lo + 32 * j); };
   auto step = [&](int j, floatx16& cur, floatx16& nxt, int koff, int koff_next, int voff, auto with_loader,
-                  int i, int kdst, int vdst) {
-    if (decltype(with_loader)::value) {
-      load_k(i + 3, kdst);
-      load_v(i + 2, vdst);
-    }
+                  int free_slot) {
+    if (decltype(with_loader)::value) feed_tile(free_slot);
     const bool in1 = j >= jq1 && j <= jp1, in2 = j >= jq2 && j <= jp2;
     if (!in1 && !in2) return;
     if (j == jq1 || (in2 && j == jq2)) {
@@ -424,47 +486,38 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   };
 
   // ---------------------------------------------------------------- main loop
-  // K tile t lives in ring slot t % 4, V tile t in slot t % 3.  At the top of iteration i the LDS
-  // holds K(i), K(i+1), V(i); K(i+2) and V(i+1) were requested during iteration i-1 and may still
-  // be in flight.  Iteration i requests K(i+3) and V(i+2) into the slots of K(i-1) and V(i-1),
-  // which no wavefront reads after the barrier that opened iteration i.  The barrier that opens
-  // iteration i+1 only waits for the older requests, so every row has a whole iteration to arrive.
-  constexpr int PER_TILE = 2 * GROUPS_PER_WAVE;  // loads per wavefront per iteration (K + V)
-  load_k(0, 0);
-  load_v(0, 0);
-  load_k(1, KTILE);
-  load_k(2, 2 * KTILE);
-  load_v(1, VTILE);
-  {
-    // Q goes through the same in-order load counter as the tile requests above, so by the time
-    // it can be scaled the first tiles have landed as well: one memory latency for the prologue.
-    const uint16_t* qrow = p.q + batch * p.q_bs + qpos * p.q_rs + hq * p.q_hs + h32 * 8;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + ks * 16);
-  }
-  scale_q();
-  tile_barrier<PER_TILE>();
+  // Stream tile t lives in ring slot t % 4 (of the K ring and of the V ring).  At the top of
+  // iteration i the LDS holds tiles i and i+1; tile i+2 was requested during iteration i-1 and
+  // may still be in flight.  Iteration i requests tile i+3 into the slot of tile i-1, which no
+  // wavefront reads after the barrier that opened iteration i.  The barrier that opens iteration
+  // i+1 only waits for the older requests, so every row has a whole iteration to arrive.
+  // At the start of a work item a wavefront has issued, after the requests for tiles 0 and 1:
+  // those for tile 2, its own Q (8 loads) and, unless it was idle, the output rows of the
+  // previous item (8 stores).  Letting PER_TILE + 8 operations pending is safe in both cases.
+  tile_barrier<PER_TILE + 8>();
   if (jq1 < 0 && jp1 >= 0) {
-    qk_block(s0, 0);
+    qk_block(s0, k0);
     settle(s0, block_max(s0), needs_mask(0), kt_lo);
 #pragma unroll
-    for (int g = 0; g < 8; ++g) ka[g] = kread(BLOCK32, g);
+    for (int g = 0; g < 8; ++g) ka[g] = kread(k0 + BLOCK32, g);
   }
-  int k0 = 0, k1 = KTILE, k2 = 2 * KTILE, k3 = 3 * KTILE;  // slots of K(i), K(i+1), K(i+2), K(i+3)
-  int v0 = 0, v1 = VTILE, v2 = 2 * VTILE;                  // slots of V(i), V(i+1), V(i+2)
   for (int i = 0; i < ntiles; ++i) {
     if (i > 0) tile_barrier<PER_TILE>();
-    step(2 * i, s0, s1, k0 + BLOCK32, k1, v0, ic<1>{}, i, k3, v2);
-    step(2 * i + 1, s1, s0, k1, k1 + BLOCK32, v0 + BLOCK32, ic<0>{}, i, 0, 0);
+    step(2 * i, s0, s1, k0 + BLOCK32, k1, k0, ic<1>{}, k3);
+    step(2 * i + 1, s1, s0, k1, k1 + BLOCK32, k0 + BLOCK32, ic<0>{}, 0);
     const int tk = k0;
     k0 = k1; k1 = k2; k2 = k3; k3 = tk;
-    const int tv = v0;
-    v0 = v1; v1 = v2; v2 = tv;
   }
 
+  // Q of the next work item is requested before the output rows of this one are stored, so that
+  // it travels while the epilogue runs (qf is dead here).
+  Where nw;
+  const bool more = locate(cw.round + 1, nw);
+  if (more) load_q(nw);
+
   // ---------------------------------------------------------------- normalise and scatter-store
-  if (!wave_active) continue;
-  const float l_tot = lane_xor32_sum(l_run);
+  if (wave_active) {
+  const float l_tot = lane_xor32_sum(l_acc[0] + l_acc[1]);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   // Lane l and lane l+32 hold the same query: per 16 head dims the lower lane has dims 0-3 and
   // 8-11, the upper one 4-7 and 12-15.  One permlane32 swap per register pair turns that into
@@ -490,6 +543,9 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
         *reinterpret_cast<u32x4*>(orow + 32 * db + 16 * g2) = pk;
       }
     }
+  }
+  if (!more) break;
+  cw = nw;
   }  // work items
 }
 
