@@ -41,7 +41,7 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   r->S = S;
   r->H = H;
   r->Hkv = Hkv;
-  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1};
+  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1};  // derived fields: geom_finish() in phases_for()
   if (domain == 0) {
     if (pattern == INTRA_LLM_SCATTER || pattern == INTRA_LLM_GATHER1) {
       if (arg0 < 1) return fail(INTRA_ERR_INVALID, "group_num must be >= 1 (got %d)", arg0);
@@ -92,6 +92,7 @@ int default_hp(int ratio) { return ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1)
 // 64-query chunks get workgroups of 2 * HP wavefronts.
 int phases_for(const Request& r, int hp, Phase ph[2]) {
   ph[0].geom = r.geom;
+  geom_finish(ph[0].geom);
   ph[0].hp = hp;
   ph[0].nw = 8;
   switch (r.kind) {
@@ -106,6 +107,7 @@ int phases_for(const Request& r, int hp, Phase ph[2]) {
   while (np % pg != 0) --pg;
   ph[0].map = MAP_IMG_PATCH;
   ph[0].geom.pg = pg;
+  geom_finish(ph[0].geom);
   ph[1] = ph[0];
   ph[1].map = MAP_IMG_SCATTER;
   ph[1].geom.text_only = 1;
@@ -345,6 +347,10 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
     p.n_pairs = dims[i].n_pairs;
     p.items_per_pair = dims[i].hgroups * dims[i].n_mblocks;
     p.n_slots = dims[i].work_items / 8;
+    p.d_items_per_pair = make_fastdiv(p.items_per_pair);
+    p.d_nbh = make_fastdiv(B * Hkv);
+    p.d_hkv = make_fastdiv(Hkv);
+    p.d_hgroups = make_fastdiv(p.hgroups);
     rc = by_map<LaunchMap>(ph[i].map, p, ph[i].hp, ph[i].nw, grid, st);
     if (rc) return rc;
   }

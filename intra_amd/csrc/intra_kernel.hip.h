@@ -67,6 +67,7 @@ struct KParams {
   int n_pairs;         // B * Hkv * n_sets
   int items_per_pair;  // hgroups * n_mblocks
   int n_slots;         // work items per XCD: ceil(n_pairs / 8) * items_per_pair
+  FastDiv d_items_per_pair, d_nbh, d_hkv, d_hgroups;  // divisions by items_per_pair, B * Hkv, Hkv, hgroups
 };
 
 constexpr int BN = 64;             // keys per tile (one barrier per tile)
@@ -148,17 +149,18 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     for (;; ++round) {
       const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
       if (slot >= p.n_slots) return false;
-      const int pair = (slot / p.items_per_pair) * 8 + xcd;
+      const int pslot = (int)fd_div(slot, p.d_items_per_pair);
+      const int pair = pslot * 8 + xcd;
       if (pair >= p.n_pairs) continue;
-      const int rem = slot % p.items_per_pair;
-      const int nbh = p.B * p.Hkv;
-      const int bh = pair % nbh;
+      const int rem = slot - pslot * p.items_per_pair;
+      const int rblk = (int)fd_div(rem, p.d_hgroups);
       w.round = round;
-      w.set = pair / nbh;
-      w.batch = bh / p.Hkv;
-      w.kvh = bh % p.Hkv;
-      w.mblk = p.n_mblocks - 1 - rem / p.hgroups;
-      w.hg = rem % p.hgroups;
+      w.set = (int)fd_div(pair, p.d_nbh);
+      const int bh = pair - w.set * (int)p.d_nbh.d;
+      w.batch = (int)fd_div(bh, p.d_hkv);
+      w.kvh = bh - w.batch * p.Hkv;
+      w.mblk = p.n_mblocks - 1 - rblk;
+      w.hg = rem - rblk * p.hgroups;
       if (w.mblk * POS >= MAP(p.geom, w.set).nq()) continue;
       return true;
     }
@@ -194,19 +196,21 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   struct Feed {
     MAP map;
     Range rg;
-    int nk, tile, round;
-    bool more;
+    int nk, tile;
+    bool more;         // false once the last work item has been requested completely
     const char *kbase, *vbase;
+    Where w;           // the work item whose tiles are being requested
+    int prev_round;    // round of the work item before it
   };
-  auto feed_for = [&](const Where& w) {
+  auto feed_for = [&](const Where& w, int prev_round) {
     const MAP map(p.geom, w.set);
-    return Feed{map, range_of(map, w.mblk), map.nk(), 0, w.round, true,
+    return Feed{map, range_of(map, w.mblk), map.nk(), 0, true,
                 reinterpret_cast<const char*>(p.k + w.batch * p.k_bs + w.kvh * p.k_hs),
-                reinterpret_cast<const char*>(p.v + w.batch * p.v_bs + w.kvh * p.v_hs)};
+                reinterpret_cast<const char*>(p.v + w.batch * p.v_bs + w.kvh * p.v_hs), w, prev_round};
   };
   Where cw;
   if (!locate(0, cw)) return;
-  Feed fd = feed_for(cw);
+  Feed fd = feed_for(cw, -1);
   auto feed_tile = [&](int slot_off) {  // request the next K and V tile of the stream into a ring slot
 #pragma unroll
     for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
@@ -219,7 +223,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     ++fd.tile;
     if (fd.tile == fd.rg.ntiles && fd.more) {
       Where w;
-      if (locate(fd.round + 1, w)) fd = feed_for(w);
+      if (locate(fd.w.round + 1, w)) fd = feed_for(w, fd.w.round);
       else fd.more = false;  // nothing left: keep requesting the (clamped) last row, nobody reads it
     }
   };
@@ -305,6 +309,15 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 
   const int hq = kvh * p.ratio + hg * HP + hw;
   const int64_t qpos = map.qpos(tq);
+  // Pin the arrival of Q here: the empty asm uses and redefines the fragments, so the compiler waits
+  // for their loads at this point (where the wait is needed anyway) and not, with a counter value
+  // that also covers the tile requests in flight, in front of every MFMA that reads them.
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    u32x4 t = __builtin_bit_cast(u32x4, qf[ks]);
+    asm volatile("" : "+v"(t));
+    qf[ks] = __builtin_bit_cast(bf16x8, t);
+  }
   if (p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
@@ -511,8 +524,11 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 
   // Q of the next work item is requested before the output rows of this one are stored, so that
   // it travels while the epilogue runs (qf is dead here).
-  Where nw;
-  const bool more = locate(cw.round + 1, nw);
+  // The loader is ahead by three tiles, so it usually knows the next work item already.
+  Where nw = fd.w;
+  bool more = true;
+  if (fd.w.round == cw.round) more = false;  // (the loader only stays on an item when it is the last)
+  else if (fd.prev_round != cw.round) more = locate(cw.round + 1, nw);
   if (more) load_q(nw);
 
   // ---------------------------------------------------------------- normalise and scatter-store

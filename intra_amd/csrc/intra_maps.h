@@ -33,6 +33,34 @@ enum IntraKind : int {
   KIND_IMG_GATHER0 = 4,
 };
 
+// Division of a non-negative int below 2^31 by a divisor fixed per launch, as multiply-high and
+// shift; the constants are worked out once on the host.
+struct FastDiv {
+  uint32_t d, mul, add, shift;
+};
+IM_HD uint32_t fd_div(uint32_t n, const FastDiv& f) {
+  return ((uint32_t)(((uint64_t)n * f.mul) >> 32) + (f.add ? n : 0u)) >> f.shift;
+}
+IM_HD uint32_t fd_mod(uint32_t n, const FastDiv& f) { return n - fd_div(n, f) * f.d; }
+inline FastDiv make_fastdiv(int d) {
+  FastDiv f;
+  f.d = (uint32_t)d;
+  if (d <= 1) {  // n / 1 = (0 + n) >> 0
+    f.d = 1;
+    f.mul = 0;
+    f.add = 1;
+    f.shift = 0;
+    return f;
+  }
+  int l = 0;
+  while ((1ll << l) < d) ++l;  // 2^(l-1) < d <= 2^l
+  // m = ceil(2^(31+l) / d) < 2^32 and floor(n * m / 2^(31+l)) = floor(n / d) for all n < 2^31
+  f.mul = (uint32_t)((((uint64_t)1 << (31 + l)) + d - 1) / d);
+  f.add = 0;
+  f.shift = (uint32_t)(l - 1);
+  return f;
+}
+
 struct IntraGeom {
   int S;         // tokens per sequence
   int G;         // LLM scatter / gather1 group count
@@ -41,7 +69,22 @@ struct IntraGeom {
   int text_len;  // image: text tokens in front of the grid
   int text_only; // image scatter: only the text queries of each group (the text rows of gather0)
   int pg;        // image gather0: 8x8 patches per set (a run of pg patches in one patch row)
+  // derived by geom_finish()
+  FastDiv dG;        // / G
+  FastDiv dWq;       // / (width / 4)
+  FastDiv dPerRow;   // / ((width / 8) / pg)
+  int g1_full;       // gather1: (S / G^2) * G
+  int g1_rem;        // gather1: S % G^2
 };
+
+inline void geom_finish(IntraGeom& ge) {
+  ge.dG = make_fastdiv(ge.G);
+  ge.dWq = make_fastdiv(ge.width / 4);
+  ge.dPerRow = make_fastdiv((ge.width / 8) / (ge.pg > 0 ? ge.pg : 1));
+  const long long gg = (long long)ge.G * ge.G;
+  ge.g1_full = (int)((ge.S / gg) * ge.G);
+  ge.g1_rem = (int)(ge.S % gg);
+}
 
 IM_HD int im_min(int a, int b) { return a < b ? a : b; }
 IM_HD int im_max(int a, int b) { return a > b ? a : b; }
@@ -56,7 +99,7 @@ struct MapLlmScatter {
   IM_HD MapLlmScatter(const IntraGeom& ge, int set) {
     G = ge.G;
     g = set;
-    n = ge.S > set ? (ge.S - set + ge.G - 1) / ge.G : 0;
+    n = ge.S > set ? (int)fd_div(ge.S - set + ge.G - 1, ge.dG) : 0;
   }
   IM_HD int nq() const { return n; }
   IM_HD int nk() const { return n; }
@@ -73,21 +116,22 @@ struct MapLlmGather1 {
   static constexpr bool kHasPrefix = false;
   IM_HD int kpre() const { return 0; }
   int G, g, n;
+  FastDiv dG;
   static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
-  static IM_HD int max_nq(const IntraGeom& ge) {
-    int gg = ge.G * ge.G;
-    return (ge.S / gg) * ge.G + im_min(ge.G, ge.S % gg);
-  }
+  static IM_HD int max_nq(const IntraGeom& ge) { return ge.g1_full + im_min(ge.G, ge.g1_rem); }
   IM_HD MapLlmGather1(const IntraGeom& ge, int set) {
     G = ge.G;
     g = set;
-    int gg = G * G;
-    int rem = ge.S % gg - G * g;  // tokens of this group in the last, partial G*G block
-    n = (ge.S / gg) * G + im_max(0, im_min(G, rem));
+    dG = ge.dG;
+    // g1_rem - G * g: tokens of this group in the last, partial G*G block
+    n = ge.g1_full + im_max(0, im_min(G, ge.g1_rem - G * g));
   }
   IM_HD int nq() const { return n; }
   IM_HD int nk() const { return n; }
-  IM_HD int qpos(int t) const { return (t / G) * (G * G) + g * G + t % G; }
+  IM_HD int qpos(int t) const {
+    const int a = (int)fd_div(t, dG);
+    return (a * G + g) * G + (t - a * G);
+  }
   IM_HD int kpos(int t) const { return qpos(t); }
   IM_HD int klo(int) const { return 0; }
   IM_HD int khi(int tq) const { return tq; }
@@ -118,6 +162,7 @@ struct MapImgScatter {
   static constexpr bool kHasPrefix = false;
   IM_HD int kpre() const { return 0; }
   int W, T, chunk, j, a, b, wq, nimg, text_only;
+  FastDiv dWq;
   static IM_HD int num_sets(const IntraGeom&) { return 8; }
   static IM_HD int max_nq(const IntraGeom& ge) {
     return ge.text_only ? ge.text_len / 8 : ge.text_len / 8 + ge.width * ge.width / 8;
@@ -132,8 +177,12 @@ struct MapImgScatter {
     wq = W / 4;
     nimg = W * W / 8;
     text_only = ge.text_only;
+    dWq = ge.dWq;
   }
-  IM_HD int imgpos(int u) const { return T + (a + 2 * (u / wq)) * W + b + 4 * (u % wq); }
+  IM_HD int imgpos(int u) const {
+    const int r = (int)fd_div(u, dWq);
+    return T + (a + 2 * r) * W + b + 4 * (u - r * wq);
+  }
   IM_HD int nq() const { return text_only ? chunk : chunk + nimg; }
   IM_HD int nk() const { return T + nimg; }
   IM_HD int qpos(int t) const { return t < chunk ? chunk * j + t : imgpos(t - chunk); }
@@ -164,9 +213,8 @@ struct MapImgPatch {
     T = ge.text_len;
     pg = ge.pg;
     np = W / 8;
-    const int per_row = np / pg;
-    R = set / per_row;
-    C0 = (set % per_row) * pg;
+    R = (int)fd_div(set, ge.dPerRow);
+    C0 = (set - R * (int)ge.dPerRow.d) * pg;
     r0 = win_start(R, np);
     cfirst = win_start(C0, np);
     nblk = (win_start(C0 + pg - 1, np) + 16 - cfirst) / 4;
