@@ -57,6 +57,26 @@ int intra_image_fwd(const void* q, const void* k, const void* v, void* o, int B,
                     const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
                     int width, int text_len, float softmax_scale, void* hip_stream);
 
+/* The same two operations with the softmax log-sum-exp as a second output: for query token t of
+ * head h, lse[b*lse_strides[0] + h*lse_strides[1] + t*lse_strides[2]] = ln sum_j exp(softmax_scale
+ * * q_t . k_j) over the keys j the pattern shows to t (fp32; strides in elements: batch, head,
+ * token).  This is the `softmax_lse` tensor that mha_fwd / mha_fwd_llm allocate and fill
+ * (csrc/flash_attn/flash_api.cpp:470,670) and that the reference's Python layer discards
+ * (intra_attn/interface.py:44,65); here it is indexed by token position, not by in-group row.
+ * It is what a backward pass or a merge of partial results over key shards needs.  Accuracy: the
+ * sum runs over the bf16-rounded weights that multiply V, so lse is within ln(1 + 2^-8) = 3.9e-3
+ * of the exact value. */
+int intra_llm_fwd_lse(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                      int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                      const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                      int group_num, int window, float softmax_scale, void* hip_stream, float* lse,
+                      const int64_t lse_strides[3]);
+int intra_image_fwd_lse(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                        int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                        const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                        int width, int text_len, float softmax_scale, void* hip_stream, float* lse,
+                        const int64_t lse_strides[3]);
+
 /* Description of the last failure on the calling thread ("" if none).  Replaces the
  * TORCH_CHECK messages of flash_api.cpp. */
 const char* intra_last_error(void);

@@ -24,6 +24,8 @@ _FWD_ARGS = [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.
 SYMBOLS = {
     "intra_llm_fwd": (ctypes.c_int, _FWD_ARGS),
     "intra_image_fwd": (ctypes.c_int, _FWD_ARGS),
+    "intra_llm_fwd_lse": (ctypes.c_int, _FWD_ARGS + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
+    "intra_image_fwd_lse": (ctypes.c_int, _FWD_ARGS + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
     "intra_last_error": (ctypes.c_char_p, []),
     "intra_version": (ctypes.c_int, []),
     "intra_plan": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.POINTER(IntraPlan)]),
@@ -44,7 +46,10 @@ def load():
         except OSError as err:
             raise ImportError(f"cannot load {LIB_PATH}: {err}") from err
         for name, (res, args) in SYMBOLS.items():
-            fn = getattr(lib, name)
+            try:
+                fn = getattr(lib, name)
+            except AttributeError as err:  # a library from an older source tree
+                raise ImportError(f"{LIB_PATH} is stale (no symbol {name}); run `python -m intra_amd.build`") from err
             fn.restype, fn.argtypes = res, args
         _lib = lib
     return _lib

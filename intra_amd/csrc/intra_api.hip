@@ -294,7 +294,8 @@ int check_strides(const char* name, const int64_t* st, int B, int S, int heads) 
 
 int run(int domain, const void* q, const void* k, const void* v, void* o, int B, int S, int H,
         int Hkv, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
-        int pattern, int arg0, int arg1, float scale, void* stream) {
+        int pattern, int arg0, int arg1, float scale, void* stream, float* lse = nullptr,
+        const int64_t* ls = nullptr, bool want_lse = false) {
   g_err[0] = 0;
   Request r;
   int rc = make_request(domain, pattern, B, S, H, Hkv, arg0, arg1, &r);
@@ -307,6 +308,15 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   if ((rc = check_strides("v", vs, B, S, Hkv))) return rc;
   if ((rc = check_strides("o", os, B, S, H))) return rc;
   if (!isfinite(scale)) return fail(INTRA_ERR_INVALID, "softmax_scale must be finite");
+  if (want_lse) {
+    if (!lse) return fail(INTRA_ERR_INVALID, "lse must be a non-null device pointer");
+    if (reinterpret_cast<uintptr_t>(lse) & 3) return fail(INTRA_ERR_INVALID, "lse must be 4-byte aligned");
+    if (!ls) return fail(INTRA_ERR_INVALID, "lse strides pointer is null");
+    for (int i = 0; i < 3; ++i)
+      if (ls[i] < 0) return fail(INTRA_ERR_INVALID, "lse stride %d is negative", i);
+    if ((B > 1 && ls[0] == 0) || (H > 1 && ls[1] == 0) || (S > 1 && ls[2] == 0))
+      return fail(INTRA_ERR_INVALID, "lse has a zero stride over a dimension larger than 1");
+  }
 
   if (ks[1] >= ((int64_t)1 << 31) || vs[1] >= ((int64_t)1 << 31))
     return fail(INTRA_ERR_UNSUPPORTED, "k / v token stride must stay below 2^31 elements");
@@ -320,6 +330,8 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.k_bs = ks[0]; p.k_rs = ks[1]; p.k_hs = ks[2];
   p.v_bs = vs[0]; p.v_rs = vs[1]; p.v_hs = vs[2];
   p.o_bs = os[0]; p.o_rs = os[1]; p.o_hs = os[2];
+  p.lse = want_lse ? lse : nullptr;
+  p.lse_bs = want_lse ? ls[0] : 0; p.lse_hs = want_lse ? ls[1] : 0; p.lse_ts = want_lse ? ls[2] : 0;
   p.B = B; p.H = H; p.Hkv = Hkv; p.ratio = H / Hkv;
   p.scale_log2 = fabsf(scale) * 1.4426950408889634f;
   if (p.scale_log2 < 1e-30f) p.scale_log2 = 1e-30f;  // scale 0: uniform weights without 0 * inf on masked scores
@@ -377,9 +389,27 @@ int intra_image_fwd(const void* q, const void* k, const void* v, void* o, int B,
              width, text_len, softmax_scale, hip_stream);
 }
 
+int intra_llm_fwd_lse(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                      int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                      const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                      int group_num, int window, float softmax_scale, void* hip_stream, float* lse,
+                      const int64_t lse_strides[3]) {
+  return run(0, q, k, v, o, B, S, H, Hkv, q_strides, k_strides, v_strides, o_strides, pattern,
+             group_num, window, softmax_scale, hip_stream, lse, lse_strides, true);
+}
+
+int intra_image_fwd_lse(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                        int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                        const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                        int width, int text_len, float softmax_scale, void* hip_stream, float* lse,
+                        const int64_t lse_strides[3]) {
+  return run(1, q, k, v, o, B, S, H, Hkv, q_strides, k_strides, v_strides, o_strides, pattern,
+             width, text_len, softmax_scale, hip_stream, lse, lse_strides, true);
+}
+
 const char* intra_last_error(void) { return g_err; }
 
-int intra_version(void) { return 100; }
+int intra_version(void) { return 200; }
 
 int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
                IntraPlan* plan) {

@@ -56,6 +56,8 @@ struct KParams {
   int64_t k_bs, k_rs, k_hs;
   int64_t v_bs, v_rs, v_hs;
   int64_t o_bs, o_rs, o_hs;
+  float* lse;          // optional (B, H, S) log-sum-exp output, or null
+  int64_t lse_bs, lse_hs, lse_ts;  // its element strides: batch, head, token
   int B, H, Hkv, ratio;
   IntraGeom geom;
   float scale_log2;    // |softmax_scale| * log2(e)
@@ -535,6 +537,8 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   if (wave_active) {
   const float l_tot = lane_xor32_sum(l_acc[0] + l_acc[1]);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (p.lse != nullptr && row_valid && h32 == 0)  // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2
+    p.lse[batch * p.lse_bs + hq * p.lse_hs + qpos * p.lse_ts] = (mref + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   // Lane l and lane l+32 hold the same query: per 16 head dims the lower lane has dims 0-3 and
   // 8-11, the upper one 4-7 and 12-15.  One permlane32 swap per register pair turns that into
   // dims 0-7 / 8-15, so each lane writes 16 contiguous bytes.

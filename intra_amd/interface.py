@@ -43,22 +43,27 @@ def _scale(q, softmax_scale):
     return q.shape[-1] ** -0.5 if softmax_scale is None else softmax_scale
 
 
-def _launch(fn, q, k, v, pattern_id, arg0, arg1, scale):
+def _launch(fn, fn_lse, q, k, v, pattern_id, arg0, arg1, scale, return_lse=False):
     out = torch.empty_like(q)
     if not _aligned(out):
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     B, S, H, _ = q.shape
+    args = [q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
+            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+            pattern_id, arg0, arg1, float(scale)]
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=q.device) if return_lse else None
     with torch.cuda.device(q.device):
         stream = torch.cuda.current_stream(q.device).cuda_stream
-        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
-                _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
-                pattern_id, arg0, arg1, float(scale), stream)
+        if return_lse:
+            rc = fn_lse(*args, stream, lse.data_ptr(), _lib.strides3(lse))
+        else:
+            rc = fn(*args, stream)
     if rc != _lib.INTRA_OK:
         raise RuntimeError(f"intra_hip: {_lib.last_error()}")
-    return out
+    return (out, lse) if return_lse else out
 
 
-def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None):
+def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None, return_lse=False):
     """Causal prefill attention for language models.
 
     pattern="scatter": token i attends to earlier tokens j with j % group_num == i % group_num.
@@ -67,15 +72,18 @@ def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_
 
     Any seqlen works for scatter and window; gather1 keeps the reference's contract of
     group_num=8 and seqlen % 64 == 0 (intra_attn/interface.py:41-42).
+
+    return_lse=True (not in the reference's signature) also returns the (batch, heads, seqlen)
+    fp32 log-sum-exp of the scaled scores of every query, as `(out, lse)`.
     """
     q, k, v = _check(q, k, v)
     if pattern == "gather1" and (group_num != 8 or q.shape[1] % (group_num * group_num)):
         raise ValueError(f"gather1 needs group_num=8 and seqlen % 64 == 0, got G={group_num}, S={q.shape[1]}")
-    return _launch(_C.intra_llm_fwd, q, k, v, LLM_PATTERNS[pattern], int(group_num), int(window),
-                   _scale(q, softmax_scale))
+    return _launch(_C.intra_llm_fwd, _C.intra_llm_fwd_lse, q, k, v, LLM_PATTERNS[pattern], int(group_num),
+                   int(window), _scale(q, softmax_scale), return_lse)
 
 
-def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None):
+def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None, return_lse=False):
     """Bidirectional attention for FLUX-style sequences: 512 text tokens followed by a
     width x width grid of image tokens.
 
@@ -84,12 +92,12 @@ def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None):
     pattern="gather0": each 8 x 8 image patch attends to a 16 x 16 window around it plus all text.
 
     Width 64 (1024 x 1024 FLUX images) and 128 (2048 x 2048), as in the reference
-    (intra_attn/interface.py:59-63).
+    (intra_attn/interface.py:59-63).  return_lse as for intra_llm_attn.
     """
     q, k, v = _check(q, k, v)
     if width not in (64, 128):
         raise ValueError("image kernels are compiled for width 64 and 128")
     if q.shape[1] != TEXT_LEN + width * width:
         raise ValueError(f"expected {TEXT_LEN} text + {width}x{width} image tokens, got {q.shape[1]}")
-    return _launch(_C.intra_image_fwd, q, k, v, IMAGE_PATTERNS[pattern], int(width), TEXT_LEN,
-                   _scale(q, softmax_scale))
+    return _launch(_C.intra_image_fwd, _C.intra_image_fwd_lse, q, k, v, IMAGE_PATTERNS[pattern], int(width),
+                   TEXT_LEN, _scale(q, softmax_scale), return_lse)

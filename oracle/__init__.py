@@ -23,7 +23,7 @@ What it restates (reference file:line) and what pins each function (tests/test_o
 Every function has at least one such independent check, so no part is "parity unpinned".
 The reference's Python file was read, not imported or run.
 """
-from .attention import masked_attention, masked_attention_rows  # noqa: F401
+from .attention import masked_attention, masked_attention_rows, masked_lse_rows  # noqa: F401
 from .masks import (TEXT_LEN, image_gather0_mask, image_scatter_mask, llm_gather1_mask,  # noqa: F401
                     llm_scatter_mask, llm_window_mask, mask_rows)
 from .pairs import pairs_per_head  # noqa: F401

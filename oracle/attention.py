@@ -37,6 +37,29 @@ def masked_attention_rows(q, k, v, mask_rows, rows=None, softmax_scale=None, chu
     return out
 
 
+def masked_lse_rows(q, k, mask_rows, rows=None, softmax_scale=None, chunk=1024):
+    """Natural log of the softmax denominator, log(sum_j exp(scale * q_i . k_j)) over the keys the
+    mask shows to row i: (B, H, len(rows)) fp32.  The reference's kernels compute this value as
+    `softmax_lse` (csrc/flash_attn/flash_api.cpp:470,670) and its Python layer drops it
+    (intra_attn/interface.py:44,65); it is one library routine, torch.logsumexp."""
+    B, S, H, D = q.shape
+    Hkv = k.shape[2]
+    rep = H // Hkv
+    scale = D ** -0.5 if softmax_scale is None else softmax_scale
+    if rows is None:
+        rows = torch.arange(S, device=q.device)
+    rows = torch.as_tensor(rows, device=q.device, dtype=torch.long)
+    kf = k.float().permute(0, 2, 3, 1)
+    out = torch.empty(B, H, rows.numel(), dtype=torch.float32, device=q.device)
+    for r0 in range(0, rows.numel(), chunk):
+        idx = rows[r0:r0 + chunk]
+        qf = q[:, idx].float().permute(0, 2, 1, 3).reshape(B, Hkv, rep, idx.numel(), D)
+        s = torch.matmul(qf, kf[:, :, None]) * scale
+        s = s.masked_fill(~mask_rows[r0:r0 + chunk].to(q.device)[None, None, None], float("-inf"))
+        out[:, :, r0:r0 + chunk] = torch.logsumexp(s, dim=-1).reshape(B, H, idx.numel())
+    return out
+
+
 def masked_attention(q, k, v, mask, softmax_scale=None, chunk=1024):
     """reference.py:78-83: q, k, v (B, S, H, D) with H % Hkv == 0; mask (S, S) bool."""
     return masked_attention_rows(q, k, v, mask, None, softmax_scale, chunk)

@@ -105,6 +105,22 @@ def test_fwd_validates_before_touching_the_gpu(lib):
     assert "expected 512 text" in _lib.last_error()
 
 
+def test_lse_entry_points_validate_their_extra_arguments(lib):
+    st = (ctypes.c_int64 * 3)(128 * 4 * 128, 4 * 128, 128)
+    ls = (ctypes.c_int64 * 3)(4 * 128, 128, 1)
+    zero = (ctypes.c_int64 * 3)(4 * 128, 0, 1)
+    ptr = 1 << 20  # never dereferenced
+    for fn, a0, a1, S in ((lib.intra_llm_fwd_lse, 8, 576, 128), (lib.intra_image_fwd_lse, 16, 8, 264)):
+        common = (ptr, ptr, ptr, ptr, 1, S, 4, 4, st, st, st, st, 0, a0, a1, 0.1, None)
+        assert fn(*common, None, ls) == 1 and "lse must be a non-null" in _lib.last_error()
+        assert fn(*common, ptr + 2, ls) == 1 and "4-byte aligned" in _lib.last_error()
+        assert fn(*common, ptr, None) == 1 and "lse strides pointer is null" in _lib.last_error()
+        assert fn(*common, ptr, zero) == 1 and "zero stride" in _lib.last_error()
+    # the shared checks still come first
+    assert lib.intra_llm_fwd_lse(None, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, st, 0, 8, 576, 0.1, None, ptr, ls) == 1
+    assert "q, k, v and o must be non-null" in _lib.last_error()
+
+
 def _model(lib, domain, pattern, S, a0, a1, hp=0, nw=0):
     count = np.zeros((S, S), dtype=np.uint8)
     rc = lib.intra_model_mask(domain, pattern, S, a0, a1, hp, nw, count.ctypes.data)

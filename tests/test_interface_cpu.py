@@ -24,11 +24,15 @@ def test_names_and_constants():
 def test_signatures_match_reference():
     import inspect
     llm = inspect.signature(intra_amd.intra_llm_attn)
-    assert list(llm.parameters) == ["q", "k", "v", "pattern", "group_num", "window", "softmax_scale"]
-    assert [p.default for p in llm.parameters.values()][3:] == ["scatter", 8, 576, None]
+    # the reference's parameters, in its order and with its defaults, come first; what this
+    # package adds follows them and defaults to the reference's behaviour
+    assert list(llm.parameters)[:7] == ["q", "k", "v", "pattern", "group_num", "window", "softmax_scale"]
+    assert [p.default for p in llm.parameters.values()][3:7] == ["scatter", 8, 576, None]
+    assert {n: p.default for n, p in list(llm.parameters.items())[7:]} == {"return_lse": False}
     img = inspect.signature(intra_amd.intra_image_attn)
-    assert list(img.parameters) == ["q", "k", "v", "pattern", "width", "softmax_scale"]
-    assert [p.default for p in img.parameters.values()][3:] == ["scatter", 64, None]
+    assert list(img.parameters)[:6] == ["q", "k", "v", "pattern", "width", "softmax_scale"]
+    assert [p.default for p in img.parameters.values()][3:6] == ["scatter", 64, None]
+    assert {n: p.default for n, p in list(img.parameters.items())[6:]} == {"return_lse": False}
 
 
 @pytest.mark.parametrize("make", [lambda: _cpu(), lambda: _cpu(dtype=torch.float16), lambda: _cpu(D=64)])

@@ -231,3 +231,30 @@ def test_attention_rows_subset_and_scale():
     sub = oracle.masked_attention_rows(q, k, v, mask[rows], rows, softmax_scale=0.05)
     assert torch.equal(sub, full[:, rows])
     assert not torch.equal(full, oracle.masked_attention(q, k, v, mask))
+
+
+def test_lse_is_the_log_of_the_softmax_denominator():
+    # float64 loop on a tiny case: lse_i = log sum_j exp(scale * q_i.k_j) over visible j, and
+    # softmax weights rebuilt from it reproduce masked_attention
+    g = torch.Generator().manual_seed(5)
+    B, S, H, Hkv, D = 1, 40, 4, 2, 128
+    q = torch.randn(B, S, H, D, generator=g)
+    k = torch.randn(B, S, Hkv, D, generator=g)
+    v = torch.randn(B, S, Hkv, D, generator=g)
+    mask = oracle.llm_scatter_mask(S, 3)
+    lse = oracle.masked_lse_rows(q, k, mask, softmax_scale=0.11)
+    assert lse.shape == (B, H, S) and lse.dtype == torch.float32
+    out = oracle.masked_attention(q, k, v, mask, softmax_scale=0.11)
+    for h in range(H):
+        for i in (0, 1, 7, 39):
+            acc, o = 0.0, torch.zeros(D, dtype=torch.float64)
+            for j in range(S):
+                if mask[i, j]:
+                    w = math.exp(0.11 * float(q[0, i, h].double() @ k[0, j, h // 2].double()))
+                    acc += w
+                    o += w * v[0, j, h // 2].double()
+            assert abs(math.log(acc) - lse[0, h, i].item()) < 1e-4
+            assert (o / acc - out[0, i, h].double()).abs().max() < 1e-4
+    rows = torch.tensor([3, 17])
+    sub = oracle.masked_lse_rows(q, k, mask[rows], rows, softmax_scale=0.11)
+    assert torch.allclose(sub, lse[:, :, rows])

@@ -224,3 +224,37 @@ def test_oracle_on_gpu_equals_oracle_on_cpu():
     a = oracle.masked_attention(q.cpu(), k.cpu(), v.cpu(), mask)
     b = oracle.masked_attention(q, k, v, mask.to(DEV)).cpu()
     assert (a.float() - b.float()).abs().max().item() <= 2 ** -8
+
+
+# fp32 log-sum-exp.  The kernel sums the bf16-rounded weights (the ones PV multiplies), each off by
+# at most 2^-8 relative, so the sum is too and the logarithm by at most ln(1 + 2^-8) = 3.9e-3.
+LSE_ATOL = 5e-3
+
+
+@pytest.mark.parametrize("kind,fn,S,H,Hkv,kw", [
+    ("llm/scatter", intra_llm_attn, 3000, 8, 2, dict(group_num=3)),
+    ("llm/gather1", intra_llm_attn, 2048, 4, 4, dict(group_num=8)),
+    ("llm/window", intra_llm_attn, 3000, 8, 2, dict(window=576)),
+    ("image/scatter", intra_image_attn, 4608, 4, 4, dict(width=64)),
+    ("image/gather0", intra_image_attn, 4608, 4, 2, dict(width=64)),
+])
+@pytest.mark.parametrize("scale", [None, -0.07])
+def test_lse_output(kind, fn, S, H, Hkv, kw, scale):
+    q, k, v = make_qkv(2, S, H, Hkv, seed=21)
+    with torch.no_grad():
+        out, lse = fn(q, k, v, kind.split("/")[1], softmax_scale=scale, return_lse=True, **kw)
+        plain = fn(q, k, v, kind.split("/")[1], softmax_scale=scale, **kw)
+    assert torch.equal(out, plain)
+    assert lse.shape == (2, H, S) and lse.dtype == torch.float32
+    mask = oracle.mask_rows(kind, S, device=DEV, **kw)
+    ref = oracle.masked_lse_rows(q, k, mask, softmax_scale=scale)
+    err = (lse - ref).abs().max().item()
+    assert err <= LSE_ATOL, f"{kind}: lse max|err|={err:.3e}"
+
+
+def test_lse_depends_on_q_and_k_only():
+    q, k, v = make_qkv(1, 2048, 4, 4, seed=22)
+    with torch.no_grad():
+        _, lse_a = intra_llm_attn(q, k, v, "scatter", group_num=2, return_lse=True)
+        _, lse_b = intra_llm_attn(q, k, torch.zeros_like(v), "scatter", group_num=2, return_lse=True)
+    assert torch.equal(lse_a, lse_b)
