@@ -31,6 +31,9 @@ enum {
 /* Pattern ids, identical to the reference's `mask` argument
  * (intra_attn/interface.py:12-13: LLM_PATTERNS, IMAGE_PATTERNS). */
 enum { INTRA_LLM_SCATTER = 0, INTRA_LLM_GATHER1 = 1, INTRA_LLM_WINDOW = 4 };
+/* Patterns of the reference's model-level experiments that its kernels do not cover (see
+ * intra_llm_fwd_ex); ids chosen here. */
+enum { INTRA_LLM_BLOCK_SCATTER = 8, INTRA_LLM_WINDOW_SINK = 9 };
 enum { INTRA_IMAGE_SCATTER = 0, INTRA_IMAGE_GATHER0 = 4 };
 
 /* Causal language-model attention.  Replaces `fwd_llm` / mha_fwd_llm
@@ -77,6 +80,22 @@ int intra_image_fwd_lse(const void* q, const void* k, const void* v, void* o, in
                         int width, int text_len, float softmax_scale, void* hip_stream, float* lse,
                         const int64_t lse_strides[3]);
 
+/* intra_llm_fwd with the two further causal patterns that the reference's LLaMA / Qwen integration
+ * runs through FlexAttention or gathered SDPA because its kernels lack them
+ * (experiments/llm/llama_intra.py:57-72, 93-110), and an optional log-sum-exp output (lse may be
+ * NULL).  Patterns 0, 1, 4 behave as in intra_llm_fwd and ignore block, offset, n_sink.
+ *   INTRA_LLM_BLOCK_SCATTER: tokens form blocks of `block` (a multiple of 64); query i in block qb
+ *     sees key j <= i in block kb iff kb % group_num == (qb + offset) % group_num, or j < n_sink,
+ *     or (offset != 0 and kb == qb).  0 <= offset < group_num, 0 <= n_sink <= block.  With
+ *     offset != 0, block must be a multiple of 256 / min(4, largest power of two in H / Hkv).
+ *   INTRA_LLM_WINDOW_SINK: query i sees key j <= i iff i - j < window or j < n_sink
+ *     (window >= 1, n_sink >= 0; group_num ignored). */
+int intra_llm_fwd_ex(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                     int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                     const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                     int group_num, int window, int block, int offset, int n_sink,
+                     float softmax_scale, void* hip_stream, float* lse, const int64_t lse_strides[3]);
+
 /* Description of the last failure on the calling thread ("" if none).  Replaces the
  * TORCH_CHECK messages of flash_api.cpp. */
 const char* intra_last_error(void);
@@ -89,7 +108,7 @@ int intra_version(void);
  * launchers (csrc/flash_attn/src/flash_fwd_launch_template.h:401-565, flash_api.cpp:408-411,
  * 611-612, 703-714). */
 typedef struct IntraPlan {
-  int kind;            /* internal pattern kind 0..4 */
+  int kind;            /* internal pattern kind 0..6 */
   int heads_per_block; /* query heads of one kv head packed into a workgroup (main launch) */
   int waves;           /* wavefronts per workgroup (main launch) */
   int pos_per_block;   /* in-set queries per workgroup (main launch) */
@@ -112,6 +131,12 @@ int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, 
  * S*S byte array the caller zeroed.  heads_per_block <= 0 means 1; waves must be 8 or <= 0. */
 int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int heads_per_block,
                      int waves, uint8_t* count);
+
+/* intra_plan / intra_model_mask for the arguments of intra_llm_fwd_ex (always 8 wavefronts). */
+int intra_plan_llm_ex(int pattern, int B, int S, int H, int Hkv, int group_num, int window,
+                      int block, int offset, int n_sink, IntraPlan* plan);
+int intra_model_mask_llm_ex(int pattern, int S, int group_num, int window, int block, int offset,
+                            int n_sink, int heads_per_block, uint8_t* count);
 
 #ifdef __cplusplus
 }

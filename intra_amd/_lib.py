@@ -26,6 +26,11 @@ SYMBOLS = {
     "intra_image_fwd": (ctypes.c_int, _FWD_ARGS),
     "intra_llm_fwd_lse": (ctypes.c_int, _FWD_ARGS + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
     "intra_image_fwd_lse": (ctypes.c_int, _FWD_ARGS + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
+    "intra_llm_fwd_ex": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 4 +
+                         [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p,
+                                               ctypes.POINTER(ctypes.c_int64)]),
+    "intra_plan_llm_ex": (ctypes.c_int, [ctypes.c_int] * 10 + [ctypes.POINTER(IntraPlan)]),
+    "intra_model_mask_llm_ex": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.c_void_p]),
     "intra_last_error": (ctypes.c_char_p, []),
     "intra_version": (ctypes.c_int, []),
     "intra_plan": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.POINTER(IntraPlan)]),

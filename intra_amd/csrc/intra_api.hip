@@ -32,7 +32,7 @@ struct Request {
 // pointers.  Mirrors the checks of intra_attn/interface.py:41-42,60-63 and
 // csrc/flash_attn/flash_api.cpp:576-612 where they still apply.
 int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
-                 Request* r) {
+                 Request* r, int block = 0, int offset = 0, int n_sink = 0, bool extended = false) {
   if (B < 1 || S < 1 || H < 1 || Hkv < 1)
     return fail(INTRA_ERR_INVALID, "B, S, H, Hkv must be positive (got %d, %d, %d, %d)", B, S, H, Hkv);
   if (H % Hkv != 0)
@@ -41,8 +41,10 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   r->S = S;
   r->H = H;
   r->Hkv = Hkv;
-  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1};  // derived fields: geom_finish() in phases_for()
+  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1, 64, 0, 0};  // derived fields: geom_finish() in phases_for()
   if (domain == 0) {
+    if (!extended && (pattern == INTRA_LLM_BLOCK_SCATTER || pattern == INTRA_LLM_WINDOW_SINK))
+      return fail(INTRA_ERR_INVALID, "unknown LLM pattern id %d (0 scatter, 1 gather1, 4 window)", pattern);
     if (pattern == INTRA_LLM_SCATTER || pattern == INTRA_LLM_GATHER1) {
       if (arg0 < 1) return fail(INTRA_ERR_INVALID, "group_num must be >= 1 (got %d)", arg0);
       if (arg0 > 32768) return fail(INTRA_ERR_INVALID, "group_num too large (%d)", arg0);
@@ -54,8 +56,29 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
                     "window must be >= 64: every 64-query block sees itself (got %d)", arg1);
       r->geom.window = arg1;
       r->kind = KIND_LLM_WINDOW;
+    } else if (pattern == INTRA_LLM_BLOCK_SCATTER) {
+      if (arg0 < 1 || arg0 > 32768) return fail(INTRA_ERR_INVALID, "group_num must be in [1, 32768] (got %d)", arg0);
+      if (block < 64 || block % 64 != 0)
+        return fail(INTRA_ERR_INVALID, "block must be a positive multiple of 64 (got %d)", block);
+      if (offset < 0 || offset >= arg0)
+        return fail(INTRA_ERR_INVALID, "offset must be in [0, group_num) (got %d)", offset);
+      if (n_sink < 0 || n_sink > block)
+        return fail(INTRA_ERR_INVALID, "n_sink must be in [0, block] (got %d)", n_sink);
+      r->geom.G = arg0;
+      r->geom.blk = block;
+      r->geom.off = offset;
+      r->geom.ns = n_sink;
+      r->kind = KIND_LLM_BLOCK_SCATTER;
+    } else if (pattern == INTRA_LLM_WINDOW_SINK) {
+      if (arg1 < 1) return fail(INTRA_ERR_INVALID, "window must be >= 1 (got %d)", arg1);
+      if (n_sink < 0) return fail(INTRA_ERR_INVALID, "n_sink must be >= 0 (got %d)", n_sink);
+      r->geom.window = arg1;
+      r->geom.ns = n_sink;
+      r->kind = KIND_LLM_WINDOW_SINK;
     } else {
-      return fail(INTRA_ERR_INVALID, "unknown LLM pattern id %d (0 scatter, 1 gather1, 4 window)", pattern);
+      return fail(INTRA_ERR_INVALID,
+                  "unknown LLM pattern id %d (0 scatter, 1 gather1, 4 window, 8 block scatter, 9 window with sinks)",
+                  pattern);
     }
   } else if (domain == 1) {
     if (pattern != INTRA_IMAGE_SCATTER && pattern != INTRA_IMAGE_GATHER0)
@@ -77,7 +100,10 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
 
 // One kernel launch: an index map, its geometry and the workgroup shape (HP query heads of one kv
 // head share a workgroup of NW wavefronts, so a row block has NW * 32 / HP in-set queries).
-enum MapId : int { MAP_LLM_SCATTER, MAP_LLM_GATHER1, MAP_LLM_WINDOW, MAP_IMG_SCATTER, MAP_IMG_PATCH };
+enum MapId : int {
+  MAP_LLM_SCATTER, MAP_LLM_GATHER1, MAP_LLM_WINDOW, MAP_IMG_SCATTER, MAP_IMG_PATCH, MAP_LLM_BLOCK_SCATTER,
+  MAP_LLM_WINDOW_SINK
+};
 struct Phase {
   int map;
   IntraGeom geom;
@@ -100,6 +126,11 @@ int phases_for(const Request& r, int hp, Phase ph[2]) {
     case KIND_LLM_GATHER1: ph[0].map = MAP_LLM_GATHER1; return 1;
     case KIND_LLM_WINDOW: ph[0].map = MAP_LLM_WINDOW; return 1;
     case KIND_IMG_SCATTER: ph[0].map = MAP_IMG_SCATTER; return 1;
+    case KIND_LLM_WINDOW_SINK: ph[0].map = MAP_LLM_WINDOW_SINK; return 1;
+    case KIND_LLM_BLOCK_SCATTER:
+      // with a stripe offset a row block (256 / hp queries) has to stay inside one query block
+      ph[0].map = MAP_LLM_BLOCK_SCATTER;
+      return (r.geom.off != 0 && r.geom.blk % (8 * 32 / hp) != 0) ? -1 : 1;
     default: break;
   }
   const int np = r.geom.width / 8;
@@ -138,12 +169,12 @@ int64_t pairs_of(const IntraGeom& ge) {
   int64_t pairs = 0;
   const int n_sets = MAP::num_sets(ge);
   for (int set = 0; set < n_sets; ++set) {
-    MAP map(ge, set);
-    const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
+    const int nq = MAP(ge, set, 0).nq();
     for (int tq = 0; tq < nq; ++tq) {
-      const int hi = im_min(map.khi(tq), nk - 1);
+      const MAP map(ge, set, tq & ~63);  // a row block of 64 queries starting at a multiple of 64
+      const int hi = im_min(map.khi(tq), map.nk() - 1), kpre = map.kpre();
       const int lo = im_max(map.klo(tq), kpre);
-      pairs += kpre + (hi >= lo ? hi - lo + 1 : 0);
+      pairs += im_min(kpre, hi + 1) + (hi >= lo ? hi - lo + 1 : 0);
     }
   }
   return pairs;
@@ -156,6 +187,8 @@ auto by_map(int map, A&&... a) {
     case MAP_LLM_GATHER1: return F<MapLlmGather1>::go(a...);
     case MAP_LLM_WINDOW: return F<MapLlmWindow>::go(a...);
     case MAP_IMG_SCATTER: return F<MapImgScatter>::go(a...);
+    case MAP_LLM_BLOCK_SCATTER: return F<MapLlmBlockScatter>::go(a...);
+    case MAP_LLM_WINDOW_SINK: return F<MapLlmWindowSink>::go(a...);
     default: return F<MapImgPatch>::go(a...);
   }
 }
@@ -163,9 +196,10 @@ template <class MAP> struct DimsOf { static PhaseDims go(const Request& r, const
 template <class MAP> struct PairsOf { static int64_t go(const IntraGeom& ge) { return pairs_of<MAP>(ge); } };
 
 // The plan describes the first (main) launch; work items and pairs are summed over all launches.
-void plan_for(const Request& r, int hp, IntraPlan* plan) {
+int plan_for(const Request& r, int hp, IntraPlan* plan) {
   Phase ph[2];
   const int n = phases_for(r, hp, ph);
+  if (n < 0) return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
   const PhaseDims d = by_map<DimsOf>(ph[0].map, r, ph[0]);
   plan->kind = r.kind;
   plan->heads_per_block = ph[0].hp;
@@ -184,6 +218,7 @@ void plan_for(const Request& r, int hp, IntraPlan* plan) {
   plan->work_items = items > 0x7fffffff ? -1 : (int)items;
   plan->grid = plan->work_items;  // upper bound; a launch uses min(its work items, 8 * (CUs / 8))
   plan->pairs_per_head = pairs;
+  return INTRA_OK;
 }
 
 // Host walk of the kernel's decomposition: sets -> row blocks -> wavefronts -> key tiles ->
@@ -195,10 +230,10 @@ void model_walk(const IntraGeom& ge, int hp, int nw, uint8_t* count) {
   const int n_sets = MAP::num_sets(ge);
   const int n_mblocks = (MAP::max_nq(ge) + pos - 1) / pos;
   for (int set = 0; set < n_sets; ++set) {
-    MAP map(ge, set);
-    const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
     for (int mblk = 0; mblk < n_mblocks; ++mblk) {
       const int t0 = mblk * pos;
+      const MAP map(ge, set, t0);
+      const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
       if (t0 >= nq) continue;
       const int t1 = im_min(t0 + pos, nq) - 1;
       const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);
@@ -295,10 +330,11 @@ int check_strides(const char* name, const int64_t* st, int B, int S, int heads) 
 int run(int domain, const void* q, const void* k, const void* v, void* o, int B, int S, int H,
         int Hkv, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
         int pattern, int arg0, int arg1, float scale, void* stream, float* lse = nullptr,
-        const int64_t* ls = nullptr, bool want_lse = false) {
+        const int64_t* ls = nullptr, bool want_lse = false, int block = 0, int offset = 0, int n_sink = 0,
+        bool extended = false) {
   g_err[0] = 0;
   Request r;
-  int rc = make_request(domain, pattern, B, S, H, Hkv, arg0, arg1, &r);
+  int rc = make_request(domain, pattern, B, S, H, Hkv, arg0, arg1, &r, block, offset, n_sink, extended);
   if (rc) return rc;
   if (!q || !k || !v || !o) return fail(INTRA_ERR_INVALID, "q, k, v and o must be non-null device pointers");
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(o))
@@ -341,6 +377,8 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
 
   Phase ph[2];
   const int n_phases = phases_for(r, default_hp(H / Hkv), ph);
+  if (n_phases < 0)
+    return fail(INTRA_ERR_UNSUPPORTED, "block scatter with an offset needs block %% 256 == 0 unless H / Hkv is even (block %% 128) or a multiple of 4 (block %% 64)");
   PhaseDims dims[2];
   for (int i = 0; i < n_phases; ++i) {
     dims[i] = by_map<DimsOf>(ph[i].map, r, ph[i]);
@@ -366,6 +404,17 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
     rc = by_map<LaunchMap>(ph[i].map, p, ph[i].hp, ph[i].nw, grid, st);
     if (rc) return rc;
   }
+  return INTRA_OK;
+}
+
+int model_mask(const Request& r, int heads_per_block, int waves, uint8_t* count) {
+  const int hp = heads_per_block > 0 ? heads_per_block : 1;
+  if ((hp != 1 && hp != 2 && hp != 4) || (waves > 0 && waves != 8))
+    return fail(INTRA_ERR_INVALID, "no kernel for heads_per_block=%d, waves=%d", hp, waves);
+  Phase ph[2];
+  const int n_phases = phases_for(r, hp, ph);
+  if (n_phases < 0) return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
+  for (int i = 0; i < n_phases; ++i) by_map<ModelWalk>(ph[i].map, ph[i].geom, ph[i].hp, ph[i].nw, count);
   return INTRA_OK;
 }
 
@@ -418,8 +467,7 @@ int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, 
   Request r;
   int rc = make_request(domain, pattern, B, S, H, Hkv, arg0, arg1, &r);
   if (rc) return rc;
-  plan_for(r, default_hp(H / Hkv), plan);
-  return INTRA_OK;
+  return plan_for(r, default_hp(H / Hkv), plan);
 }
 
 int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int heads_per_block,
@@ -429,13 +477,37 @@ int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int hea
   Request r;
   int rc = make_request(domain, pattern, 1, S, 1, 1, arg0, arg1, &r);
   if (rc) return rc;
-  const int hp = heads_per_block > 0 ? heads_per_block : 1;
-  if ((hp != 1 && hp != 2 && hp != 4) || (waves > 0 && waves != 8))
-    return fail(INTRA_ERR_INVALID, "no kernel for heads_per_block=%d, waves=%d", hp, waves);
-  Phase ph[2];
-  const int n_phases = phases_for(r, hp, ph);
-  for (int i = 0; i < n_phases; ++i) by_map<ModelWalk>(ph[i].map, ph[i].geom, ph[i].hp, ph[i].nw, count);
-  return INTRA_OK;
+  return model_mask(r, heads_per_block, waves, count);
+}
+
+int intra_llm_fwd_ex(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                     int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                     const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                     int group_num, int window, int block, int offset, int n_sink,
+                     float softmax_scale, void* hip_stream, float* lse, const int64_t lse_strides[3]) {
+  return run(0, q, k, v, o, B, S, H, Hkv, q_strides, k_strides, v_strides, o_strides, pattern,
+             group_num, window, softmax_scale, hip_stream, lse, lse_strides, lse != nullptr, block, offset,
+             n_sink, true);
+}
+
+int intra_plan_llm_ex(int pattern, int B, int S, int H, int Hkv, int group_num, int window,
+                      int block, int offset, int n_sink, IntraPlan* plan) {
+  g_err[0] = 0;
+  if (!plan) return fail(INTRA_ERR_INVALID, "plan pointer is null");
+  Request r;
+  int rc = make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true);
+  if (rc) return rc;
+  return plan_for(r, default_hp(H / Hkv), plan);
+}
+
+int intra_model_mask_llm_ex(int pattern, int S, int group_num, int window, int block, int offset,
+                            int n_sink, int heads_per_block, uint8_t* count) {
+  g_err[0] = 0;
+  if (!count) return fail(INTRA_ERR_INVALID, "count pointer is null");
+  Request r;
+  int rc = make_request(0, pattern, 1, S, 1, 1, group_num, window, &r, block, offset, n_sink, true);
+  if (rc) return rc;
+  return model_mask(r, heads_per_block, 8, count);
 }
 
 }  // extern "C"

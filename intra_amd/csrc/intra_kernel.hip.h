@@ -163,7 +163,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
       w.kvh = bh - w.batch * p.Hkv;
       w.mblk = p.n_mblocks - 1 - rblk;
       w.hg = rem - rblk * p.hgroups;
-      if (w.mblk * POS >= MAP(p.geom, w.set).nq()) continue;
+      if (w.mblk * POS >= MAP(p.geom, w.set, w.mblk * POS).nq()) continue;
       return true;
     }
   };
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     int prev_round;    // round of the work item before it
   };
   auto feed_for = [&](const Where& w, int prev_round) {
-    const MAP map(p.geom, w.set);
+    const MAP map(p.geom, w.set, w.mblk * POS);
     return Feed{map, range_of(map, w.mblk), map.nk(), 0, true,
                 reinterpret_cast<const char*>(p.k + w.batch * p.k_bs + w.kvh * p.k_hs),
                 reinterpret_cast<const char*>(p.v + w.batch * p.v_bs + w.kvh * p.v_hs), w, prev_round};
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   bf16x8 qf[8];
   // this lane's query row of a work item (clamped to the last row of the row block)
   auto q_row = [&](const Where& w) {
-    const MAP map(p.geom, w.set);
+    const MAP map(p.geom, w.set, w.mblk * POS);
     const int t1 = im_min(w.mblk * POS + POS, map.nq()) - 1;
     const int tq = im_min(w.mblk * POS + (wave / HP) * 32 + l32, t1);
     const int hq = w.kvh * p.ratio + w.hg * HP + wave % HP;
@@ -275,10 +275,10 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 
   for (;;) {
   const int set = cw.set, batch = cw.batch, kvh = cw.kvh, mblk = cw.mblk, hg = cw.hg;
-  const MAP map(p.geom, set);
+  const int t0 = mblk * POS;
+  const MAP map(p.geom, set, t0);
   const int nq = map.nq();
   const int nk = map.nk();
-  const int t0 = mblk * POS;
   const int t1 = im_min(t0 + POS, nq) - 1;
   const int kpre = map.kpre();  // keys every query of the set sees (0 if none)
   const Range rg = range_of(map, mblk);
@@ -298,12 +298,13 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   // and, for maps with a prefix, the prefix blocks in front of it.
   int bw_lo = __builtin_amdgcn_readfirstlane((wb.w_lo - kt_lo) / 32);
   int bw_hi = __builtin_amdgcn_readfirstlane((wb.w_hi - kt_lo) / 32);
-  int bp_hi = MAP::kHasPrefix ? (kpre - 1) / 32 : -1;  // last prefix block
-  if (!wave_active) {
-    bw_lo = 1;
+  // last prefix block it looks at (a causal bound may end the prefix early)
+  int bp_hi = MAP::kHasPrefix && kpre > 0 ? __builtin_amdgcn_readfirstlane(im_min(kpre - 1, wb.w_hi) / 32) : -1;
+  if (!wave_active || wb.w_lo > wb.w_hi) {  // no own range: an empty run of steps
+    bw_lo = 2;
     bw_hi = 0;
-    bp_hi = -1;
   }
+  if (!wave_active) bp_hi = -1;
   wb.f_lo = __builtin_amdgcn_readfirstlane(wb.f_lo);
   wb.f_hi = __builtin_amdgcn_readfirstlane(wb.f_hi);
   wb.w_lo = __builtin_amdgcn_readfirstlane(wb.w_lo);

@@ -3,10 +3,13 @@
 //
 // A "set" is a group of query tokens that share one packed key list.  Inside a set, queries are
 // numbered tq = 0..nq-1 and keys tk = 0..nk-1 ("in-set indices"); qpos()/kpos() turn an in-set
-// index into a token position of the (B, S, H, 128) tensors.  Query tq attends exactly the keys
-// klo(tq) <= tk <= min(khi(tq), nk-1).  klo and khi are non-decreasing in tq for every pattern,
-// which is what lets a wavefront classify a whole 32x32 score block as skipped / unmasked /
-// partially masked from the bounds of its first and last query alone.
+// index into a token position of the (B, S, H, 128) tensors.  With hi = min(khi(tq), nk-1), query
+// tq attends exactly the keys tk <= hi that are either below kpre() (a prefix every query of the
+// set looks at, 0 for most maps) or at least klo(tq).  klo and khi are non-decreasing in tq for
+// every pattern, which is what lets a wavefront classify a whole 32x32 score block as skipped /
+// unmasked / partially masked from the bounds of its first and last query alone.
+// A map is built for one row block of a set (constructor argument t0 = its first in-set query):
+// the key numbering of some patterns depends on where the row block sits.
 //
 // Semantics follow the dense-mask specification of the reference:
 //   LLM scatter   intra_attn/reference.py:14-17    index map csrc/flash_attn/src/gmem_tile.h:511,656
@@ -14,6 +17,8 @@
 //   LLM window    intra_attn/reference.py:27-32    csrc/flash_attn/src/flash_fwd_kernel.h:7008
 //   image scatter intra_attn/reference.py:36-53    gmem_tile.h:286-340,388-389
 //   image gather0 intra_attn/reference.py:56-74    gmem_tile.h:1220-1294,1334-1373
+//   LLM block scatter (blocks, stripe offset, own block, sinks)  experiments/llm/llama_intra.py:93-110
+//   LLM per-token window with sinks                             experiments/llm/llama_intra.py:57-72
 // The maps here are re-derived from those predicates; nothing is shared with the reference code.
 #pragma once
 #include <stdint.h>
@@ -31,6 +36,8 @@ enum IntraKind : int {
   KIND_LLM_WINDOW = 2,
   KIND_IMG_SCATTER = 3,
   KIND_IMG_GATHER0 = 4,
+  KIND_LLM_BLOCK_SCATTER = 5,
+  KIND_LLM_WINDOW_SINK = 6,
 };
 
 // Division of a non-negative int below 2^31 by a divisor fixed per launch, as multiply-high and
@@ -69,10 +76,14 @@ struct IntraGeom {
   int text_len;  // image: text tokens in front of the grid
   int text_only; // image scatter: only the text queries of each group (the text rows of gather0)
   int pg;        // image gather0: 8x8 patches per set (a run of pg patches in one patch row)
+  int blk;       // LLM block scatter: tokens per block
+  int off;       // LLM block scatter: stripe offset, 0 <= off < G
+  int ns;        // LLM block scatter / window with sinks: leading tokens every query sees
   // derived by geom_finish()
   FastDiv dG;        // / G
   FastDiv dWq;       // / (width / 4)
   FastDiv dPerRow;   // / ((width / 8) / pg)
+  FastDiv dBlk;      // / blk
   int g1_full;       // gather1: (S / G^2) * G
   int g1_rem;        // gather1: S % G^2
 };
@@ -81,6 +92,7 @@ inline void geom_finish(IntraGeom& ge) {
   ge.dG = make_fastdiv(ge.G);
   ge.dWq = make_fastdiv(ge.width / 4);
   ge.dPerRow = make_fastdiv((ge.width / 8) / (ge.pg > 0 ? ge.pg : 1));
+  ge.dBlk = make_fastdiv(ge.blk);
   const long long gg = (long long)ge.G * ge.G;
   ge.g1_full = (int)((ge.S / gg) * ge.G);
   ge.g1_rem = (int)(ge.S % gg);
@@ -96,7 +108,7 @@ struct MapLlmScatter {
   int G, g, n;
   static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
   static IM_HD int max_nq(const IntraGeom& ge) { return (ge.S + ge.G - 1) / ge.G; }
-  IM_HD MapLlmScatter(const IntraGeom& ge, int set) {
+  IM_HD MapLlmScatter(const IntraGeom& ge, int set, int /*t0*/) {
     G = ge.G;
     g = set;
     n = ge.S > set ? (int)fd_div(ge.S - set + ge.G - 1, ge.dG) : 0;
@@ -119,7 +131,7 @@ struct MapLlmGather1 {
   FastDiv dG;
   static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
   static IM_HD int max_nq(const IntraGeom& ge) { return ge.g1_full + im_min(ge.G, ge.g1_rem); }
-  IM_HD MapLlmGather1(const IntraGeom& ge, int set) {
+  IM_HD MapLlmGather1(const IntraGeom& ge, int set, int /*t0*/) {
     G = ge.G;
     g = set;
     dG = ge.dG;
@@ -144,7 +156,7 @@ struct MapLlmWindow {
   int S, lookback;
   static IM_HD int num_sets(const IntraGeom&) { return 1; }
   static IM_HD int max_nq(const IntraGeom& ge) { return ge.S; }
-  IM_HD MapLlmWindow(const IntraGeom& ge, int) {
+  IM_HD MapLlmWindow(const IntraGeom& ge, int, int /*t0*/) {
     S = ge.S;
     lookback = ge.window - 64;
   }
@@ -167,7 +179,7 @@ struct MapImgScatter {
   static IM_HD int max_nq(const IntraGeom& ge) {
     return ge.text_only ? ge.text_len / 8 : ge.text_len / 8 + ge.width * ge.width / 8;
   }
-  IM_HD MapImgScatter(const IntraGeom& ge, int set) {
+  IM_HD MapImgScatter(const IntraGeom& ge, int set, int /*t0*/) {
     W = ge.width;
     T = ge.text_len;
     chunk = T / 8;
@@ -208,7 +220,7 @@ struct MapImgPatch {
   }
   static IM_HD int num_sets(const IntraGeom& ge) { return (ge.width / 8) * ((ge.width / 8) / ge.pg); }
   static IM_HD int max_nq(const IntraGeom& ge) { return 64 * ge.pg; }
-  IM_HD MapImgPatch(const IntraGeom& ge, int set) {
+  IM_HD MapImgPatch(const IntraGeom& ge, int set, int /*t0*/) {
     W = ge.width;
     T = ge.text_len;
     pg = ge.pg;
@@ -235,11 +247,98 @@ struct MapImgPatch {
   IM_HD int khi(int tq) const { return klo(tq) + 255; }
 };
 
+// ------- LLM block scatter: blocks of blk tokens, block b in group b % G.  A query of block qb sees,
+// causally, the blocks of group (qb + off) % G, the first ns tokens ("sinks", ns <= blk) and, when
+// off != 0, its own block.  The key list of a row block is numbered
+//   [sinks, unless the next part starts with them] [blocks of the target group] [own block, off != 0]
+// where the own block follows the last target block in front of it, so that every query sees the
+// contiguous range 0..khi.  With off != 0 the numbering depends on the query block, hence row
+// blocks must not straddle query blocks (the host picks the row-block size accordingly).
+struct MapLlmBlockScatter {
+  static constexpr bool kHasPrefix = false;
+  IM_HD int kpre() const { return 0; }
+  int G, blk, g, gt, off, n, E, own_base, own_len, qb;
+  FastDiv dBlk;
+  static IM_HD int group_size(const IntraGeom& ge, int g) {  // tokens in blocks b = g (mod G)
+    const int nb = (int)fd_div(ge.S, ge.dBlk);               // full blocks
+    const int tail = ge.S - nb * ge.blk;
+    const int full = nb > g ? (int)fd_div(nb - 1 - g, ge.dG) + 1 : 0;
+    return full * ge.blk + ((tail > 0 && (int)fd_mod(nb, ge.dG) == g) ? tail : 0);
+  }
+  static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
+  static IM_HD int max_nq(const IntraGeom& ge) {
+    int m = 0;
+    for (int g = 0; g < ge.G; ++g) m = im_max(m, group_size(ge, g));
+    return m;
+  }
+  IM_HD MapLlmBlockScatter(const IntraGeom& ge, int set, int t0) {
+    G = ge.G;
+    blk = ge.blk;
+    off = ge.off;
+    dBlk = ge.dBlk;
+    g = set;
+    gt = g + off >= G ? g + off - G : g + off;  // target group
+    n = group_size(ge, g);
+    const int a = (int)fd_div(t0, dBlk);         // query block of the row block, within the group
+    qb = a * G + g;
+    const int ns = im_min(ge.ns, ge.S);
+    own_len = im_max(0, im_min(blk, ge.S - qb * blk));  // tokens the own block really has
+    if (off == 0) {
+      E = g == 0 ? 0 : ns;
+      own_base = 0x7fffffff;                     // no own-block part
+    } else {
+      E = (gt == 0 || qb == 0) ? 0 : ns;         // block 0 is in front already / is the own block
+      own_base = E + (a + (gt < g ? 1 : 0)) * blk;
+    }
+  }
+  IM_HD int nq() const { return n; }
+  IM_HD int nk() const { return off == 0 ? E + n : own_base + own_len; }
+  IM_HD int qpos(int t) const {
+    const int a = (int)fd_div(t, dBlk);
+    return (a * G + g) * blk + (t - a * blk);
+  }
+  IM_HD int kpos(int t) const {
+    if (t < E) return t;
+    if (t >= own_base) return qb * blk + (t - own_base);
+    const int c = t - E;
+    const int m = (int)fd_div(c, dBlk);
+    return (m * G + gt) * blk + (c - m * blk);
+  }
+  IM_HD int klo(int) const { return 0; }
+  IM_HD int khi(int tq) const {
+    if (off == 0) return E + tq;
+    return own_base + (tq - (int)fd_div(tq, dBlk) * blk);
+  }
+};
+
+// ------- LLM per-token sliding window with sinks: query i sees the keys j <= i with i - j < window
+// or j < ns.  One set; the key list of a row block is numbered [sinks][positions wlo, wlo+1, ...]
+// with wlo = the first position outside the sinks that its first query sees, so that tiles start
+// at the window and not at position 0.
+struct MapLlmWindowSink {
+  static constexpr bool kHasPrefix = true;
+  int S, window, ns, wlo;
+  static IM_HD int num_sets(const IntraGeom&) { return 1; }
+  static IM_HD int max_nq(const IntraGeom& ge) { return ge.S; }
+  IM_HD MapLlmWindowSink(const IntraGeom& ge, int, int t0) {
+    S = ge.S;
+    window = ge.window;
+    ns = im_min(ge.ns, ge.S);
+    wlo = im_max(t0 - window + 1, ns);
+  }
+  IM_HD int nq() const { return S; }
+  IM_HD int nk() const { return ns + (S - wlo); }
+  IM_HD int kpre() const { return ns; }
+  IM_HD int qpos(int t) const { return t; }
+  IM_HD int kpos(int t) const { return t < ns ? t : wlo + (t - ns); }
+  IM_HD int klo(int tq) const { return ns + im_max(tq - window + 1, wlo) - wlo; }
+  IM_HD int khi(int tq) const { return tq < ns ? tq : ns + (tq - wlo); }
+};
+
 // --------------------------------------------------------------------------- block classification
-// A wavefront owns the queries wq0..wq_last of a set.  Query tq sees the keys below kpre() (the
-// prefix, if the map has one) and klo(tq)..min(khi(tq), nk-1).
+// A wavefront owns the queries wq0..wq_last of a set.
 struct WaveBounds {
-  int w_lo, w_hi;  // union of the key ranges of the wavefront's queries
+  int w_lo, w_hi;  // union of the [klo, hi] ranges of the wavefront's queries
   int f_lo, f_hi;  // intersection of them
 };
 
@@ -256,9 +355,9 @@ IM_HD WaveBounds wave_bounds(const MAP& map, int wq0, int wq_last) {
 
 // Does the wavefront look at the 32 keys sb_lo..sb_lo+31 at all, and can it skip the mask?
 IM_HD bool block_wanted(const WaveBounds& wb, int kpre, int sb_lo) {
-  return sb_lo < kpre || (sb_lo <= wb.w_hi && sb_lo + 31 >= wb.w_lo);
+  return sb_lo <= wb.w_hi && (sb_lo < kpre || sb_lo + 31 >= wb.w_lo);
 }
 IM_HD bool block_unmasked(const WaveBounds& wb, int kpre, int sb_lo) {
-  return sb_lo + 31 < kpre || (sb_lo >= kpre && sb_lo >= wb.f_lo && sb_lo + 31 <= wb.f_hi);
+  return sb_lo + 31 <= wb.f_hi && (sb_lo + 31 < kpre || (sb_lo >= kpre && sb_lo >= wb.f_lo));
 }
-IM_HD bool key_visible(int key, int kpre, int lo, int hi) { return key < kpre || (key >= lo && key <= hi); }
+IM_HD bool key_visible(int key, int kpre, int lo, int hi) { return key <= hi && (key < kpre || key >= lo); }

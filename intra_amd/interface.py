@@ -15,6 +15,9 @@ _C = _lib.load()
 
 LLM_PATTERNS = {"scatter": 0, "gather1": 1, "window": 4}
 IMAGE_PATTERNS = {"scatter": 0, "gather0": 4}
+# Patterns of the reference's LLaMA / Qwen integration that its kernels do not have
+# (experiments/llm/llama_intra.py:57-72,93-110); they run through intra_llm_fwd_ex.
+EXTRA_LLM_PATTERNS = {"block_scatter": 8, "window_sink": 9}
 TEXT_LEN = 512
 
 
@@ -63,7 +66,26 @@ def _launch(fn, fn_lse, q, k, v, pattern_id, arg0, arg1, scale, return_lse=False
     return (out, lse) if return_lse else out
 
 
-def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None, return_lse=False):
+def _launch_ex(q, k, v, pattern_id, group_num, window, block, offset, n_sink, scale, return_lse):
+    out = torch.empty_like(q)
+    if not _aligned(out):
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    B, S, H, _ = q.shape
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=q.device) if return_lse else None
+    with torch.cuda.device(q.device):
+        stream = torch.cuda.current_stream(q.device).cuda_stream
+        rc = _C.intra_llm_fwd_ex(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
+                                 _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                                 pattern_id, group_num, window, block, offset, n_sink, float(scale), stream,
+                                 lse.data_ptr() if return_lse else None,
+                                 _lib.strides3(lse) if return_lse else None)
+    if rc != _lib.INTRA_OK:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
+    return (out, lse) if return_lse else out
+
+
+def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None, return_lse=False,
+                   block=256, offset=0, n_sink=0):
     """Causal prefill attention for language models.
 
     pattern="scatter": token i attends to earlier tokens j with j % group_num == i % group_num.
@@ -73,12 +95,23 @@ def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_
     Any seqlen works for scatter and window; gather1 keeps the reference's contract of
     group_num=8 and seqlen % 64 == 0 (intra_attn/interface.py:41-42).
 
-    return_lse=True (not in the reference's signature) also returns the (batch, heads, seqlen)
-    fp32 log-sum-exp of the scaled scores of every query, as `(out, lse)`.
+    Not in the reference's signature:
+    return_lse=True also returns the (batch, heads, seqlen) fp32 log-sum-exp of the scaled scores
+    of every query, as `(out, lse)`.
+    pattern="block_scatter": tokens form blocks of `block` (a multiple of 64), block b in group
+        b % group_num; a query block qb reads the earlier blocks of group (qb + offset) % group_num
+        and itself where it is in that group or offset != 0, plus the first n_sink tokens.
+    pattern="window_sink": query i sees keys j <= i with i - j < window or j < n_sink.
+    These two are the Scatter and window layers of the reference's model integration
+    (experiments/llm/llama_intra.py; its LLaMA setting is group_num=2, block=256, offset 0 / 1,
+    window=575, n_sink=64).
     """
     q, k, v = _check(q, k, v)
     if pattern == "gather1" and (group_num != 8 or q.shape[1] % (group_num * group_num)):
         raise ValueError(f"gather1 needs group_num=8 and seqlen % 64 == 0, got G={group_num}, S={q.shape[1]}")
+    if pattern in EXTRA_LLM_PATTERNS:
+        return _launch_ex(q, k, v, EXTRA_LLM_PATTERNS[pattern], int(group_num), int(window), int(block),
+                          int(offset), int(n_sink), _scale(q, softmax_scale), return_lse)
     return _launch(_C.intra_llm_fwd, _C.intra_llm_fwd_lse, q, k, v, LLM_PATTERNS[pattern], int(group_num),
                    int(window), _scale(q, softmax_scale), return_lse)
 

@@ -35,6 +35,27 @@ def llm_window_mask(S, window=576, block=64, device=None, rows=None):
     return (k <= q) & (k >= start)
 
 
+def llm_block_scatter_mask(S, group_num=2, block=256, offset=0, n_sink=0, device=None, rows=None):
+    """experiments/llm/llama_intra.py:98-110 (mask_mod of _scatter_block_mask): blocks of `block`
+    tokens, block b in group b % G; a query block qb reads, causally, the key blocks of group
+    (qb + offset) % G, with offset != 0 also its own block, and the first n_sink tokens."""
+    q, k = _qk(S, rows, device)
+    qb, kb = q // block, k // block
+    vis = (kb % group_num) == ((qb + offset) % group_num)
+    if offset:
+        vis = vis | (kb == qb)
+    if n_sink:
+        vis = vis | (k < n_sink)
+    return (k <= q) & vis
+
+
+def llm_window_sink_mask(S, window=575, n_sink=0, device=None, rows=None):
+    """experiments/llm/llama_intra.py:62-72 (mask_mod of _sliding_block_mask): causal, and the key
+    is among the last `window` positions up to the query or among the first n_sink tokens."""
+    q, k = _qk(S, rows, device)
+    return (k <= q) & ((q - k < window) | (k < n_sink))
+
+
 def _image_group(pos, width, text_len):
     """reference.py:36-46: text token t -> t // (text_len/8); grid token (r, c) -> (r%2)*4 + c%4."""
     p = (pos - text_len).clamp(min=0)
@@ -69,13 +90,18 @@ def image_gather0_mask(width, text_len=TEXT_LEN, patch=8, window=16, device=None
 
 def mask_rows(kind, S, rows=None, device=None, **kw):
     """Dispatch by the API's names: kind in {"llm/scatter", "llm/gather1", "llm/window",
-    "image/scatter", "image/gather0"}."""
+    "llm/block_scatter", "llm/window_sink", "image/scatter", "image/gather0"}."""
     if kind == "llm/scatter":
         return llm_scatter_mask(S, kw.get("group_num", 8), device, rows)
     if kind == "llm/gather1":
         return llm_gather1_mask(S, kw.get("group_num", 8), device, rows)
     if kind == "llm/window":
         return llm_window_mask(S, kw.get("window", 576), 64, device, rows)
+    if kind == "llm/block_scatter":
+        return llm_block_scatter_mask(S, kw.get("group_num", 2), kw.get("block", 256), kw.get("offset", 0),
+                                      kw.get("n_sink", 0), device, rows)
+    if kind == "llm/window_sink":
+        return llm_window_sink_mask(S, kw.get("window", 575), kw.get("n_sink", 0), device, rows)
     width = kw.get("width", 64)
     text_len = kw.get("text_len", TEXT_LEN)
     assert S == text_len + width * width

@@ -160,3 +160,65 @@ def test_model_rejects_unknown_shape(lib):
     count = np.zeros((64, 64), dtype=np.uint8)
     assert lib.intra_model_mask(0, 0, 64, 8, 576, 3, 8, count.ctypes.data) == 1
     assert "no kernel" in _lib.last_error()
+
+
+# ------------------------------------------------------------------ block scatter / window with sinks
+EX_CASES = \
+    [(S, "llm/block_scatter", 8, dict(group_num=G, block=blk, offset=off, n_sink=ns))
+     for S in (1, 64, 200, 1000, 1537) for (G, blk, off, ns) in
+     ((2, 256, 0, 0), (2, 256, 1, 64), (2, 256, 0, 64), (3, 64, 2, 10), (3, 128, 1, 128), (4, 64, 0, 33),
+      (1, 64, 0, 0), (2, 512, 1, 0))] + \
+    [(S, "llm/window_sink", 9, dict(window=W, n_sink=ns))
+     for S in (1, 63, 200, 1000, 1300) for (W, ns) in
+     ((575, 64), (575, 0), (1, 0), (1, 5), (64, 64), (100, 37), (5000, 64), (300, 700))]
+
+
+def _model_ex(lib, pattern, S, hp, group_num=2, window=575, block=256, offset=0, n_sink=0):
+    count = np.zeros((S, S), dtype=np.uint8)
+    rc = lib.intra_model_mask_llm_ex(pattern, S, group_num, window, block, offset, n_sink, hp, count.ctypes.data)
+    return rc, torch.from_numpy(count)
+
+
+@pytest.mark.parametrize("S,kind,pattern,kw", EX_CASES)
+@pytest.mark.parametrize("hp", [1, 2, 4])
+def test_kernel_decomposition_equals_mask_llm_ex(lib, S, kind, pattern, kw, hp):
+    rc, count = _model_ex(lib, pattern, S, hp, **kw)
+    if kw.get("offset", 0) and kw["block"] % (256 // hp):  # row blocks would straddle query blocks
+        assert rc == _lib.INTRA_ERR_UNSUPPORTED
+        return
+    assert rc == 0, _lib.last_error()
+    want = oracle.mask_rows(kind, S, **kw)
+    assert torch.equal(count, want.to(torch.uint8)), f"{kind} {kw} hp={hp}: kernel walk differs from the mask"
+
+
+@pytest.mark.parametrize("S,kind,pattern,kw", EX_CASES[::3])
+def test_plan_ex_pair_counts(lib, S, kind, pattern, kw):
+    p = _lib.IntraPlan()
+    rc = lib.intra_plan_llm_ex(pattern, 1, S, 8, 2, kw.get("group_num", 2), kw.get("window", 575),
+                               kw.get("block", 256), kw.get("offset", 0), kw.get("n_sink", 0), ctypes.byref(p))
+    assert rc == 0, _lib.last_error()
+    assert p.pairs_per_head == oracle.pairs_per_head(kind, S, **kw) == int(oracle.mask_rows(kind, S, **kw).sum())
+
+
+def test_ex_argument_checks(lib):
+    p = _lib.IntraPlan()
+    bad = [((8, 1, 512, 4, 4, 2, 575, 100, 0, 0), "block must be a positive multiple of 64"),
+           ((8, 1, 512, 4, 4, 2, 575, 256, 2, 0), "offset must be in [0, group_num)"),
+           ((8, 1, 512, 4, 4, 2, 575, 256, 0, 300), "n_sink must be in [0, block]"),
+           ((9, 1, 512, 4, 4, 2, 0, 256, 0, 0), "window must be >= 1"),
+           ((9, 1, 512, 4, 4, 2, 575, 256, 0, -1), "n_sink must be >= 0"),
+           ((7, 1, 512, 4, 4, 2, 575, 256, 0, 0), "unknown LLM pattern")]
+    for args, text in bad:
+        assert lib.intra_plan_llm_ex(*args, ctypes.byref(p)) == _lib.INTRA_ERR_INVALID
+        assert text in _lib.last_error()
+    # a stripe offset needs row blocks inside one query block: 64-token blocks with 1 q head per kv head
+    assert lib.intra_plan_llm_ex(8, 1, 512, 4, 4, 2, 575, 64, 1, 0, ctypes.byref(p)) == _lib.INTRA_ERR_UNSUPPORTED
+    assert lib.intra_plan_llm_ex(8, 1, 512, 16, 4, 2, 575, 64, 1, 0, ctypes.byref(p)) == 0
+    assert (p.heads_per_block, p.pos_per_block) == (4, 64)
+    assert lib.intra_plan_llm_ex(8, 1, 512, 8, 4, 2, 575, 128, 1, 0, ctypes.byref(p)) == 0
+    assert (p.heads_per_block, p.pos_per_block) == (2, 128)
+    # the old patterns pass through and ignore the extra arguments
+    q = _lib.IntraPlan()
+    assert lib.intra_plan_llm_ex(0, 1, 32768, 32, 8, 8, 576, 0, 0, 0, ctypes.byref(p)) == 0
+    assert lib.intra_plan(0, 0, 1, 32768, 32, 8, 8, 576, ctypes.byref(q)) == 0
+    assert (p.work_items, p.pairs_per_head) == (q.work_items, q.pairs_per_head)

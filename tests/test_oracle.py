@@ -258,3 +258,102 @@ def test_lse_is_the_log_of_the_softmax_denominator():
     rows = torch.tensor([3, 17])
     sub = oracle.masked_lse_rows(q, k, mask[rows], rows, softmax_scale=0.11)
     assert torch.allclose(sub, lse[:, :, rows])
+
+
+# ------------------------------------------------------------------ block scatter / window with sinks
+def _loop_block_scatter(S, G, blk, off, ns):
+    m = torch.zeros(S, S, dtype=torch.bool)
+    for i in range(S):
+        for j in range(i + 1):
+            same_class = (j // blk) % G == ((i // blk) + off) % G
+            m[i, j] = same_class or (off != 0 and j // blk == i // blk) or j < ns
+    return m
+
+
+@pytest.mark.parametrize("S,G,blk,off,ns", [(70, 2, 16, 0, 0), (70, 2, 16, 1, 5), (90, 3, 8, 2, 8), (50, 4, 4, 0, 3)])
+def test_block_scatter_mask_brute_force(S, G, blk, off, ns):
+    assert torch.equal(masks.llm_block_scatter_mask(S, G, blk, off, ns), _loop_block_scatter(S, G, blk, off, ns))
+
+
+def test_block_scatter_reduces_to_scatter_and_gather1():
+    for S, G in ((100, 2), (257, 3), (1000, 8)):
+        assert torch.equal(masks.llm_block_scatter_mask(S, G, 1, 0, 0), masks.llm_scatter_mask(S, G))
+        assert torch.equal(masks.llm_block_scatter_mask(S, G, G, 0, 0), masks.llm_gather1_mask(S, G))
+    assert torch.equal(masks.llm_block_scatter_mask(300, 1, 64, 0, 0), torch.ones(300, 300).tril().bool())
+
+
+def test_block_scatter_offsets_partition_the_earlier_blocks():
+    # every key block in front of a query block is read at exactly one offset; the own block is read
+    # at every offset; sinks add nothing once block 0 is visible
+    S, G, blk = 640, 4, 64
+    ms = [masks.llm_block_scatter_mask(S, G, blk, off, 0) for off in range(G)]
+    total = sum(m.to(torch.int32) for m in ms)
+    qb = torch.arange(S)[:, None] // blk
+    kb = torch.arange(S)[None, :] // blk
+    causal = torch.ones(S, S).tril().bool()
+    assert torch.equal(total[(kb < qb)], torch.ones_like(total[(kb < qb)]))
+    assert torch.equal(total[(kb == qb) & causal], torch.full_like(total[(kb == qb) & causal], G))
+    assert int(total[~causal].sum()) == 0
+    for off in range(G):
+        with_sinks = masks.llm_block_scatter_mask(S, G, blk, off, 48)
+        extra = with_sinks & ~ms[off]
+        assert bool((extra.nonzero()[:, 1] < 48).all()) and torch.equal(with_sinks | ms[off], with_sinks)
+        assert bool(with_sinks.any(dim=1).all())  # no empty row
+
+
+def test_block_scatter_equals_gathered_group_attention_with_sinks():
+    """The reference builds the same layer a second way (llama_intra.py:124-165): per group, gather
+    the group's tokens, put the sink tokens in front of the key list (dropping them from the
+    group's own part) and run causal attention in original positions.  Restated here with plain
+    softmax; it must agree with masked attention under llm_block_scatter_mask at offset 0."""
+    g = torch.Generator().manual_seed(9)
+    B, S, H, Hkv, D, G, blk, ns = 1, 300, 2, 1, 128, 2, 64, 20
+    q = torch.randn(B, S, H, D, generator=g)
+    k = torch.randn(B, S, Hkv, D, generator=g)
+    v = torch.randn(B, S, Hkv, D, generator=g)
+    ref = oracle.masked_attention(q, k, v, masks.llm_block_scatter_mask(S, G, blk, 0, ns), softmax_scale=0.1)
+    out = torch.zeros_like(q)
+    pos = torch.arange(S)
+    gid = (pos // blk) % G
+    for grp in range(G):
+        idx = pos[gid == grp]
+        kv = torch.cat([pos[:ns], idx[idx >= ns]])
+        allowed = kv[None, :] <= idx[:, None]
+        for h in range(H):
+            s = (q[0, idx, h].double() @ k[0, kv, 0].double().T) * 0.1
+            s = s.masked_fill(~allowed, float("-inf"))
+            out[0, idx, h] = (torch.softmax(s, -1) @ v[0, kv, 0].double()).float()
+    assert (out - ref).abs().max() < 1e-5
+
+
+def test_window_sink_mask_special_cases_and_counts():
+    S = 300
+    tril = torch.ones(S, S).tril().bool()
+    assert torch.equal(masks.llm_window_sink_mask(S, S, 0), tril)
+    assert torch.equal(masks.llm_window_sink_mask(S, 5000, 7), tril)
+    assert torch.equal(masks.llm_window_sink_mask(S, 1, 0), torch.eye(S).bool())
+    for W, ns in ((575, 64), (100, 37), (64, 64), (1, 5), (17, 0)):
+        m = masks.llm_window_sink_mask(S, W, ns)
+        assert not bool((m & ~tril).any())
+        rows = m.sum(1)
+        want = torch.tensor([min(i + 1, W) + max(0, min(ns, i + 1 - W)) for i in range(S)])
+        assert torch.equal(rows, want)
+        # the window part is a band, the rest sits in the first ns columns
+        i = torch.arange(S)[:, None]
+        j = torch.arange(S)[None, :]
+        band = (j <= i) & (j > i - W)
+        assert torch.equal(m & band, band) and bool(((m & ~band).nonzero()[:, 1] < ns).all())
+    m = masks.llm_window_sink_mask(200, 96, 4)
+    assert m[130, 35] and not m[130, 34] and m[130, 3] and not m[130, 4] and m[2, 2] and not m[2, 3]
+
+
+def test_new_pair_counts_match_masks():
+    for S in (1, 100, 777):
+        for kw in (dict(group_num=2, block=64, offset=0, n_sink=0), dict(group_num=2, block=64, offset=1, n_sink=20),
+                   dict(group_num=3, block=128, offset=2, n_sink=128), dict(group_num=4, block=64, offset=0, n_sink=9)):
+            assert pairs.pairs_per_head("llm/block_scatter", S, **kw) == int(oracle.mask_rows("llm/block_scatter", S, **kw).sum())
+        for kw in (dict(window=575, n_sink=64), dict(window=10, n_sink=3), dict(window=1, n_sink=0)):
+            assert pairs.pairs_per_head("llm/window_sink", S, **kw) == int(oracle.mask_rows("llm/window_sink", S, **kw).sum())
+    rows = torch.tensor([0, 5, 99])
+    assert torch.equal(oracle.mask_rows("llm/window_sink", 100, rows=rows, window=10, n_sink=3),
+                       masks.llm_window_sink_mask(100, 10, 3)[rows])
