@@ -22,7 +22,7 @@ if ROOT not in sys.path:
 PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU; AMD publishes it as 2.5 PFLOP/s dense
 # HBM bytes per launch at S=32768 measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/); None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {32768: 971e6}
+MEASURED_TRAFFIC_BYTES = {32768: 793e6}
 
 
 def main():
@@ -116,7 +116,7 @@ def main():
     if not args.no_cpu:
         # Bounded sample of the same problem: evenly spaced query rows of all heads against all
         # keys through the dense-mask fp32 path, on the host cores.
-        n_rows = 1024 if S >= 8192 else S
+        n_rows = 4096 if S >= 8192 else S  # about 10 s on 16 host cores
         rows_c = torch.arange(0, S, S // n_rows)[:n_rows]
         mask_c = oracle.llm_scatter_mask(S, G, rows=rows_c)
         cores = torch.get_num_threads()

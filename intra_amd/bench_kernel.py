@@ -41,6 +41,15 @@ def pairs(domain, pattern, B, S, H, Hkv, a0, a1):
     return plan.pairs_per_head
 
 
+def pairs_ex(pattern, B, S, H, Hkv, group_num, window, block, offset, n_sink):
+    import ctypes
+    plan = _lib.IntraPlan()
+    rc = _lib.load().intra_plan_llm_ex(pattern, B, S, H, Hkv, group_num, window, block, offset, n_sink,
+                                       ctypes.byref(plan))
+    assert rc == 0, _lib.last_error()
+    return plan.pairs_per_head
+
+
 def dense_sdpa(q, k, v, causal):
     q, k, v = (x.transpose(1, 2) for x in (q, k, v))
     return F.scaled_dot_product_attention(q, k, v, is_causal=causal, enable_gqa=q.shape[1] != k.shape[1])
@@ -89,6 +98,26 @@ def bench_llm(args):
                     else:
                         intra_llm_attn(ql, kl, vl, "window", window=576)
             r["g2s4_32layer_run_ms"] = round(median_ms(stack, 2, max(3, args.iters // 10)), 3)
+        if args.model_patterns:
+            # the layers the reference's model integration really runs in its g2s4 LLaMA setting
+            # (experiments/llm/llama_intra.py:16-18): block Scatter with 2 groups of 256-token
+            # blocks, stripe offset 0 / 1, 64 sink tokens; per-token window 575 with 64 sinks
+            for off in (0, 1):
+                kw = dict(group_num=2, block=256, offset=off, n_sink=64)
+                ms = median_ms(lambda: intra_llm_attn(q, k, v, "block_scatter", **kw), args.warmup, args.iters)
+                r[f"block_scatter_g2_b256_off{off}_sink64"] = entry(ms, pairs_ex(8, B, S, H, Hkv, 2, 575, 256, off, 64), B, H)
+            ms = median_ms(lambda: intra_llm_attn(q, k, v, "window_sink", window=575, n_sink=64), args.warmup, args.iters)
+            r["window575_sink64"] = entry(ms, pairs_ex(9, B, S, H, Hkv, 2, 575, 256, 0, 64), B, H)
+            layers = [qkv(B, S, H, Hkv, seed=i) for i in range(4)]
+
+            def model_stack():
+                for i in range(32):
+                    ql, kl, vl = layers[i % 4]
+                    if i % 8 == 0:
+                        intra_llm_attn(ql, kl, vl, "block_scatter", group_num=2, block=256, offset=(i // 8) % 2, n_sink=64)
+                    else:
+                        intra_llm_attn(ql, kl, vl, "window_sink", window=575, n_sink=64)
+            r["g2s4_model_32layer_run_ms"] = round(median_ms(model_stack, 2, max(3, args.iters // 10)), 3)
         rows.append(r)
         print(json.dumps(r), flush=True)
     return rows
@@ -125,6 +154,8 @@ def main():
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--iters", type=int, default=50)
     p.add_argument("--dense", action="store_true", help="also time torch SDPA on the dense problem")
+    p.add_argument("--model-patterns", action="store_true",
+                   help="llm: also time block Scatter and window-with-sinks layers (g2s4 model setting)")
     p.add_argument("--out", help="optional JSON output path")
     args = p.parse_args()
     args.seqlens = [int(x) for x in args.seqlens.split(",")]
