@@ -208,7 +208,7 @@ def test_attention_vs_float64_loops():
 
 
 @pytest.mark.parametrize("B,S,H,Hkv,kind,kw", [
-    (1, 1024, 4, 1, "llm/scatter", dict(group_num=8)),   # BASELINE config 1
+    (1, 1024, 4, 1, "llm/scatter", dict(group_num=8)),   # the reference's CPU-runnable configuration
     (2, 300, 6, 2, "llm/window", dict(window=100)),
     (1, 320, 3, 3, "image/gather0", dict(width=16, text_len=64))])
 def test_attention_vs_torch_sdpa(B, S, H, Hkv, kind, kw):

@@ -1,5 +1,5 @@
 """Parity of every kernel against the fp32 dense-mask oracle, through the Python API and the
-C ABI behind it.  Case matrix of the reference's tests/test_kernel.py:33-51 plus the BASELINE
+C ABI behind it.  Case matrix of the reference's tests/test_kernel.py:33-51 plus the headline
 shapes, ragged / tiny / strided inputs and size-independent properties at full length.
 
 Tolerance: max-abs error <= 1.6e-2 on bf16 outputs (README.md:68-69 of the reference; its own
@@ -310,3 +310,31 @@ def test_llm_ex_full_length_row_subset(pattern, kw):
         out = intra_llm_attn(q, k, v, pattern, **kw)
     rows = _row_subset(S, 512, seed=35)
     check(out, q, k, v, f"llm/{pattern}", rows=rows, **kw)
+
+
+def test_calls_can_be_captured_in_a_graph_and_replayed():
+    """The library allocates nothing and only enqueues kernels on the given stream, so a call can
+    be recorded into a HIP graph.  Every replay (with new inputs copied into the captured tensors
+    and ordinary eager work in between) must reproduce the eager result."""
+    q, k, v = make_qkv(1, 4608, 8, 8, seed=41)
+    calls = [lambda q, k, v: intra_llm_attn(q, k, v, "scatter", group_num=8),
+             lambda q, k, v: intra_llm_attn(q, k, v, "window_sink", window=575, n_sink=64),
+             lambda q, k, v: intra_image_attn(q, k, v, "gather0", 64)]  # two launches
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for fn in calls:  # warm up outside the capture
+                fn(q, k, v)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = [fn(q, k, v) for fn in calls]
+        for rep in range(3):
+            q2, k2, v2 = make_qkv(1, 4608, 8, 8, seed=50 + rep)
+            q.copy_(q2), k.copy_(k2), v.copy_(v2)
+            graph.replay()
+            torch.cuda.synchronize()
+            for fn, got in zip(calls, outs):
+                want = fn(q, k, v)  # eager, on the same (updated) tensors
+                assert torch.equal(got, want), f"replay {rep} differs from the eager call"
