@@ -1,7 +1,8 @@
 // Forward sparse-attention kernel for gfx950 (MI355X): one template for all five INTRA patterns.
 //
 // Replaces the reference's five CUDA kernels (csrc/flash_attn/src/flash_fwd_kernel.h:3970-6158
-// with their loaders in gmem_tile.h) by one wave64/MFMA design:
+// with their loaders in gmem_tile.h) by one wave64/MFMA design, which also runs the block-level
+// Scatter and window-with-sinks layers of experiments/llm/llama_intra.py:
 //
 //  * A workgroup of NW wavefronts owns a row block of one set: POS = NW*32/HP consecutive in-set
 //    queries of HP query heads that share one KV head (GQA packing), so every gathered K/V tile
@@ -17,11 +18,12 @@
 //    block j+1 and the 8 PV MFMAs of block j, with the softmax VALU work of block j spread over
 //    both phases and every LDS operand read issued a whole phase (8 MFMAs) ahead.
 //  * K/V rows are gathered from HBM straight into LDS (global_load_lds_dwordx4, 16 lanes per
-//    256-byte row, no register staging), three tiles ahead for K and two for V; one barrier per
-//    64-key tile, which only waits for the requests of the previous iteration.  An LDS tile is
-//    16 groups of 4 rows with an XOR chunk swizzle inside the group and 16 bytes of padding
-//    between groups, so the row-per-lane K reads and the 4-row transposing V reads are both free
-//    of bank conflicts.
+//    256-byte row, no register staging), three tiles ahead; one barrier per 64-key tile, which
+//    only waits for the requests of the previous iteration.  The tiles of all work items of a
+//    workgroup form one stream through the ring, so the first tiles of a work item arrive while
+//    the previous one still computes.  An LDS tile is 16 groups of 4 rows with an XOR chunk
+//    swizzle inside the group and 16 bytes of padding between groups, so the row-per-lane K reads
+//    and the 4-row transposing V reads are both free of bank conflicts.
 //  * The softmax reference stays 0 (weights exp2(score*c), exact after normalisation because
 //    numerator and denominator share it) unless a block maximum leaves the +-60 exponent band;
 //    then the query is re-centred and O rescaled.  No per-block rescale in the common case.
