@@ -117,7 +117,7 @@ typedef struct IntraPlan {
   int work_items;      /* row blocks to process, all launches (a multiple of 8: padded per XCD) */
   int grid;            /* upper bound of workgroups launched: min(work_items, CUs of the device) */
   int lds_bytes;       /* LDS per workgroup */
-  int launches;        /* kernel launches per call: 1, or 2 for image gather0 (grid rows, text rows) */
+  int launches;        /* kernel launches per call (1 for every pattern of this build) */
   int64_t pairs_per_head; /* unmasked (query, key) pairs per query head and batch */
 } IntraPlan;
 

@@ -101,8 +101,8 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
 // One kernel launch: an index map, its geometry and the workgroup shape (HP query heads of one kv
 // head share a workgroup of NW wavefronts, so a row block has NW * 32 / HP in-set queries).
 enum MapId : int {
-  MAP_LLM_SCATTER, MAP_LLM_GATHER1, MAP_LLM_WINDOW, MAP_IMG_SCATTER, MAP_IMG_PATCH, MAP_LLM_BLOCK_SCATTER,
-  MAP_LLM_WINDOW_SINK
+  MAP_LLM_SCATTER, MAP_LLM_GATHER1, MAP_LLM_WINDOW, MAP_IMG_SCATTER, MAP_LLM_BLOCK_SCATTER,
+  MAP_LLM_WINDOW_SINK, MAP_IMG_GATHER0
 };
 struct Phase {
   int map;
@@ -112,10 +112,9 @@ struct Phase {
 
 int default_hp(int ratio) { return ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1); }
 
-// Every pattern is one launch of 8-wavefront workgroups, except image gather0: its grid queries
-// run as sets of `pg` neighbouring 8x8 patches (as many as fit into a row block), its text
-// queries - which see what the scatter pattern shows them - as text-only scatter sets, whose
-// 64-query chunks get workgroups of 2 * HP wavefronts.
+// Every pattern is one launch of 8-wavefront workgroups.  Image gather0 runs its grid queries as
+// sets of `pg` neighbouring 8x8 patches (as many as fit into a row block) and its text queries -
+// which see what the scatter pattern shows them - as text-only scatter sets of the same launch.
 int phases_for(const Request& r, int hp, Phase ph[2]) {
   ph[0].geom = r.geom;
   geom_finish(ph[0].geom);
@@ -136,14 +135,10 @@ int phases_for(const Request& r, int hp, Phase ph[2]) {
   const int np = r.geom.width / 8;
   int pg = im_max(1, (8 * 32 / hp) / 64);
   while (np % pg != 0) --pg;
-  ph[0].map = MAP_IMG_PATCH;
+  ph[0].map = MAP_IMG_GATHER0;
   ph[0].geom.pg = pg;
   geom_finish(ph[0].geom);
-  ph[1] = ph[0];
-  ph[1].map = MAP_IMG_SCATTER;
-  ph[1].geom.text_only = 1;
-  ph[1].nw = 2 * hp;
-  return 2;
+  return 1;
 }
 
 struct PhaseDims {
@@ -189,7 +184,7 @@ auto by_map(int map, A&&... a) {
     case MAP_IMG_SCATTER: return F<MapImgScatter>::go(a...);
     case MAP_LLM_BLOCK_SCATTER: return F<MapLlmBlockScatter>::go(a...);
     case MAP_LLM_WINDOW_SINK: return F<MapLlmWindowSink>::go(a...);
-    default: return F<MapImgPatch>::go(a...);
+    default: return F<MapImgGather0>::go(a...);
   }
 }
 template <class MAP> struct DimsOf { static PhaseDims go(const Request& r, const Phase& ph) { return dims_of<MAP>(r, ph); } };
@@ -303,10 +298,6 @@ struct LaunchMap {
         case 2: return launch<MAP, 2, 8>(p, grid, stream);
         case 1: return launch<MAP, 1, 8>(p, grid, stream);
       }
-    }
-    if (std::is_same<MAP, MapImgScatter>::value) {  // 64-query text chunks of gather0
-      if (hp == 2 && nw == 4) return launch<MapImgScatter, 2, 4>(p, grid, stream);
-      if (hp == 1 && nw == 2) return launch<MapImgScatter, 1, 2>(p, grid, stream);
     }
     return fail(INTRA_ERR_UNSUPPORTED, "no kernel for heads_per_block=%d, waves=%d", hp, nw);
   }

@@ -179,7 +179,7 @@ struct MapImgScatter {
   static IM_HD int max_nq(const IntraGeom& ge) {
     return ge.text_only ? ge.text_len / 8 : ge.text_len / 8 + ge.width * ge.width / 8;
   }
-  IM_HD MapImgScatter(const IntraGeom& ge, int set, int /*t0*/) {
+  IM_HD MapImgScatter(const IntraGeom& ge, int set, int /*t0*/, int only_text = -1) {
     W = ge.width;
     T = ge.text_len;
     chunk = T / 8;
@@ -188,7 +188,7 @@ struct MapImgScatter {
     b = set & 3;
     wq = W / 4;
     nimg = W * W / 8;
-    text_only = ge.text_only;
+    text_only = only_text < 0 ? ge.text_only : only_text;
     dWq = ge.dWq;
   }
   IM_HD int imgpos(int u) const {
@@ -208,8 +208,8 @@ struct MapImgScatter {
 // row, so that the text keys (a prefix every query sees) and most of the window keys are shared.
 // The window keys of the set are the union of the patches' windows, cut into blocks of 4 grid
 // columns x 16 grid rows = 64 keys; window starts are multiples of 4, so a patch sees exactly 4
-// consecutive blocks.  The text queries of gather0 keep their scatter rows and are computed with
-// MapImgScatter in text_only mode.
+// consecutive blocks.  The text queries of gather0 keep their scatter rows (MapImgScatter in
+// text_only mode); MapImgGather0 below puts both kinds of sets into one launch.
 struct MapImgPatch {
   static constexpr bool kHasPrefix = true;
   int W, T, pg, np, R, C0, r0, cfirst, nblk;
@@ -245,6 +245,26 @@ struct MapImgPatch {
   }
   IM_HD int klo(int tq) const { return T + 16 * (win_start(C0 + (tq >> 6), np) - cfirst); }
   IM_HD int khi(int tq) const { return klo(tq) + 255; }
+};
+
+// ---- image gather0, all rows: sets 0..7 are the text-only scatter sets (the longest work items,
+// so they come first), sets 8.. the patch runs.
+struct MapImgGather0 {
+  static constexpr bool kHasPrefix = true;
+  bool is_text;
+  MapImgScatter sc;
+  MapImgPatch pa;
+  static IM_HD int num_sets(const IntraGeom& ge) { return 8 + MapImgPatch::num_sets(ge); }
+  static IM_HD int max_nq(const IntraGeom& ge) { return im_max(ge.text_len / 8, MapImgPatch::max_nq(ge)); }
+  IM_HD MapImgGather0(const IntraGeom& ge, int set, int t0)
+      : is_text(set < 8), sc(ge, set < 8 ? set : 0, t0, 1), pa(ge, set < 8 ? 0 : set - 8, t0) {}
+  IM_HD int nq() const { return is_text ? sc.nq() : pa.nq(); }
+  IM_HD int nk() const { return is_text ? sc.nk() : pa.nk(); }
+  IM_HD int kpre() const { return is_text ? 0 : pa.kpre(); }
+  IM_HD int qpos(int t) const { return is_text ? sc.qpos(t) : pa.qpos(t); }
+  IM_HD int kpos(int t) const { return is_text ? sc.kpos(t) : pa.kpos(t); }
+  IM_HD int klo(int tq) const { return is_text ? 0 : pa.klo(tq); }
+  IM_HD int khi(int tq) const { return is_text ? sc.khi(tq) : pa.khi(tq); }
 };
 
 // ------- LLM block scatter: blocks of blk tokens, block b in group b % G.  A query of block qb sees,

@@ -38,16 +38,14 @@ def test_plan_headline(lib):
     assert p.pairs_per_head == 67125248 and 0 < p.lds_bytes <= 160 * 1024
 
 
-def test_plan_gather0_is_two_launches(lib):
-    # grid rows: sets of 4 / 2 / 1 neighbouring 8x8 patches; text rows: 8 text-only scatter sets
+def test_plan_gather0_sets(lib):
+    # one launch: 8 text-only scatter sets, then sets of 4 / 2 / 1 neighbouring 8x8 patches
     for H, Hkv, hp, pg in ((24, 24, 1, 4), (16, 8, 2, 2), (32, 8, 4, 1)):
         rc, p = _plan(lib, 1, 4, 1, 16896, H, Hkv, 128, 512)
-        assert rc == 0 and p.launches == 2
+        assert rc == 0 and p.launches == 1
         assert (p.heads_per_block, p.waves, p.pos_per_block) == (hp, 8, 256 // hp)
-        assert (p.n_sets, p.n_mblocks) == (16 * 16 // pg, 1)
-        patch_items = 8 * -(-Hkv * p.n_sets // 8) * (H // Hkv // hp)
-        text_items = 8 * -(-Hkv * 8 // 8) * (H // Hkv // hp)
-        assert p.work_items == patch_items + text_items
+        assert (p.n_sets, p.n_mblocks) == (8 + 16 * 16 // pg, 1)
+        assert p.work_items == 8 * -(-Hkv * p.n_sets // 8) * (H // Hkv // hp)
     rc, p = _plan(lib, 1, 0, 1, 16896, 24, 24, 128, 512)
     assert rc == 0 and p.launches == 1
 
