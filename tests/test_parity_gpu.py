@@ -338,3 +338,41 @@ def test_calls_can_be_captured_in_a_graph_and_replayed():
             for fn, got in zip(calls, outs):
                 want = fn(q, k, v)  # eager, on the same (updated) tensors
                 assert torch.equal(got, want), f"replay {rep} differs from the eager call"
+
+
+def _random_cases(n, seed):
+    import random
+    rnd = random.Random(seed)
+    heads = [(4, 4), (4, 2), (8, 2), (4, 1), (16, 4), (3, 3), (6, 3)]
+    cases = []
+    for _ in range(n):
+        H, Hkv = rnd.choice(heads)
+        B = rnd.choice([1, 1, 2])
+        S = rnd.choice([rnd.randint(1, 300), rnd.randint(300, 3000), 64 * rnd.randint(1, 40)])
+        kind = rnd.choice(["scatter", "gather1", "window", "block_scatter", "window_sink"])
+        if kind == "scatter":
+            kw = dict(group_num=rnd.choice([1, 2, 3, 5, 8, 13]))
+        elif kind == "gather1":
+            S = 64 * max(1, S // 64)
+            kw = dict(group_num=8)
+        elif kind == "window":
+            kw = dict(window=rnd.choice([64, 65, 128, 576, 1000, 4000]))
+        elif kind == "block_scatter":
+            G = rnd.choice([1, 2, 3, 4])
+            blk = 256 * rnd.choice([1, 1, 2]) if (H // Hkv) % 4 else 64 * rnd.choice([1, 2, 4, 8])
+            kw = dict(group_num=G, block=blk, offset=rnd.randrange(G), n_sink=rnd.choice([0, 1, 64, blk]))
+        else:
+            kw = dict(window=rnd.choice([1, 2, 63, 64, 575, 2000]), n_sink=rnd.choice([0, 1, 64, 100, 700]))
+        cases.append((kind, B, S, H, Hkv, kw, rnd.choice([None, None, 0.05, -0.11])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(48, seed=2024), ids=lambda c: f"{c[0]}-S{c[2]}-H{c[3]}/{c[4]}")
+def test_random_llm_shapes(case):
+    kind, B, S, H, Hkv, kw, scale = case
+    q, k, v = make_qkv(B, S, H, Hkv, seed=S + H)
+    with torch.no_grad():
+        out, lse = intra_llm_attn(q, k, v, kind, softmax_scale=scale, return_lse=True, **kw)
+    check(out, q, k, v, f"llm/{kind}", scale=scale, rtol=2.0 ** -7, **kw)
+    ref = oracle.masked_lse_rows(q, k, oracle.mask_rows(f"llm/{kind}", S, device=DEV, **kw), softmax_scale=scale)
+    assert (lse - ref).abs().max().item() <= LSE_ATOL
