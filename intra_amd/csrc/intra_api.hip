@@ -41,7 +41,7 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   r->S = S;
   r->H = H;
   r->Hkv = Hkv;
-  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1, 64, 0, 0};  // derived fields: geom_finish() in phases_for()
+  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1, 64, 0, 0};  // derived fields: geom_finish() in shape_for()
   if (domain == 0) {
     if (!extended && (pattern == INTRA_LLM_BLOCK_SCATTER || pattern == INTRA_LLM_WINDOW_SINK))
       return fail(INTRA_ERR_INVALID, "unknown LLM pattern id %d (0 scatter, 1 gather1, 4 window)", pattern);
@@ -98,13 +98,13 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   return INTRA_OK;
 }
 
-// One kernel launch: an index map, its geometry and the workgroup shape (HP query heads of one kv
-// head share a workgroup of NW wavefronts, so a row block has NW * 32 / HP in-set queries).
+// The kernel launch of a request: an index map, its geometry and the workgroup shape (HP query heads
+// of one kv head share a workgroup of NW wavefronts, so a row block has NW * 32 / HP in-set queries).
 enum MapId : int {
   MAP_LLM_SCATTER, MAP_LLM_GATHER1, MAP_LLM_WINDOW, MAP_IMG_SCATTER, MAP_LLM_BLOCK_SCATTER,
   MAP_LLM_WINDOW_SINK, MAP_IMG_GATHER0
 };
-struct Phase {
+struct Shape {
   int map;
   IntraGeom geom;
   int hp, nw;
@@ -115,39 +115,40 @@ int default_hp(int ratio) { return ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1)
 // Every pattern is one launch of 8-wavefront workgroups.  Image gather0 runs its grid queries as
 // sets of `pg` neighbouring 8x8 patches (as many as fit into a row block) and its text queries -
 // which see what the scatter pattern shows them - as text-only scatter sets of the same launch.
-int phases_for(const Request& r, int hp, Phase ph[2]) {
-  ph[0].geom = r.geom;
-  geom_finish(ph[0].geom);
-  ph[0].hp = hp;
-  ph[0].nw = 8;
+bool shape_for(const Request& r, int hp, Shape* ph) {  // false: no kernel shape fits
+  ph->geom = r.geom;
+  ph->hp = hp;
+  ph->nw = 8;
   switch (r.kind) {
-    case KIND_LLM_SCATTER: ph[0].map = MAP_LLM_SCATTER; return 1;
-    case KIND_LLM_GATHER1: ph[0].map = MAP_LLM_GATHER1; return 1;
-    case KIND_LLM_WINDOW: ph[0].map = MAP_LLM_WINDOW; return 1;
-    case KIND_IMG_SCATTER: ph[0].map = MAP_IMG_SCATTER; return 1;
-    case KIND_LLM_WINDOW_SINK: ph[0].map = MAP_LLM_WINDOW_SINK; return 1;
+    case KIND_LLM_SCATTER: ph->map = MAP_LLM_SCATTER; break;
+    case KIND_LLM_GATHER1: ph->map = MAP_LLM_GATHER1; break;
+    case KIND_LLM_WINDOW: ph->map = MAP_LLM_WINDOW; break;
+    case KIND_IMG_SCATTER: ph->map = MAP_IMG_SCATTER; break;
+    case KIND_LLM_WINDOW_SINK: ph->map = MAP_LLM_WINDOW_SINK; break;
     case KIND_LLM_BLOCK_SCATTER:
       // with a stripe offset a row block (256 / hp queries) has to stay inside one query block
-      ph[0].map = MAP_LLM_BLOCK_SCATTER;
-      return (r.geom.off != 0 && r.geom.blk % (8 * 32 / hp) != 0) ? -1 : 1;
-    default: break;
+      ph->map = MAP_LLM_BLOCK_SCATTER;
+      if (r.geom.off != 0 && r.geom.blk % (8 * 32 / hp) != 0) return false;
+      break;
+    default: {
+      const int np = r.geom.width / 8;
+      int pg = im_max(1, (8 * 32 / hp) / 64);
+      while (np % pg != 0) --pg;
+      ph->map = MAP_IMG_GATHER0;
+      ph->geom.pg = pg;
+    }
   }
-  const int np = r.geom.width / 8;
-  int pg = im_max(1, (8 * 32 / hp) / 64);
-  while (np % pg != 0) --pg;
-  ph[0].map = MAP_IMG_GATHER0;
-  ph[0].geom.pg = pg;
-  geom_finish(ph[0].geom);
-  return 1;
+  geom_finish(ph->geom);
+  return true;
 }
 
-struct PhaseDims {
+struct LaunchDims {
   int pos, n_sets, n_mblocks, hgroups, n_pairs, work_items;
 };
 
 template <class MAP>
-PhaseDims dims_of(const Request& r, const Phase& ph) {
-  PhaseDims d;
+LaunchDims dims_of(const Request& r, const Shape& ph) {
+  LaunchDims d;
   d.pos = ph.nw * 32 / ph.hp;
   d.n_sets = MAP::num_sets(ph.geom);
   d.n_mblocks = (MAP::max_nq(ph.geom) + d.pos - 1) / d.pos;
@@ -187,32 +188,25 @@ auto by_map(int map, A&&... a) {
     default: return F<MapImgGather0>::go(a...);
   }
 }
-template <class MAP> struct DimsOf { static PhaseDims go(const Request& r, const Phase& ph) { return dims_of<MAP>(r, ph); } };
+template <class MAP> struct DimsOf { static LaunchDims go(const Request& r, const Shape& ph) { return dims_of<MAP>(r, ph); } };
 template <class MAP> struct PairsOf { static int64_t go(const IntraGeom& ge) { return pairs_of<MAP>(ge); } };
 
-// The plan describes the first (main) launch; work items and pairs are summed over all launches.
 int plan_for(const Request& r, int hp, IntraPlan* plan) {
-  Phase ph[2];
-  const int n = phases_for(r, hp, ph);
-  if (n < 0) return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
-  const PhaseDims d = by_map<DimsOf>(ph[0].map, r, ph[0]);
+  Shape ph;
+  if (!shape_for(r, hp, &ph))
+    return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
+  const LaunchDims d = by_map<DimsOf>(ph.map, r, ph);
   plan->kind = r.kind;
-  plan->heads_per_block = ph[0].hp;
-  plan->waves = ph[0].nw;
+  plan->heads_per_block = ph.hp;
+  plan->waves = ph.nw;
   plan->pos_per_block = d.pos;
   plan->n_sets = d.n_sets;
   plan->n_mblocks = d.n_mblocks;
-  plan->launches = n;
+  plan->launches = 1;
   plan->lds_bytes = intra::LDS_BYTES;
-  int64_t items = 0, pairs = 0;
-  for (int i = 0; i < n; ++i) {
-    const PhaseDims di = by_map<DimsOf>(ph[i].map, r, ph[i]);
-    items = (di.work_items < 0 || items < 0) ? -1 : items + di.work_items;
-    pairs += by_map<PairsOf>(ph[i].map, ph[i].geom);
-  }
-  plan->work_items = items > 0x7fffffff ? -1 : (int)items;
+  plan->work_items = d.work_items;
   plan->grid = plan->work_items;  // upper bound; a launch uses min(its work items, 8 * (CUs / 8))
-  plan->pairs_per_head = pairs;
+  plan->pairs_per_head = by_map<PairsOf>(ph.map, ph.geom);
   return INTRA_OK;
 }
 
@@ -366,46 +360,37 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.k_rs_bytes = (uint32_t)(ks[1] * 2);
   p.v_rs_bytes = (uint32_t)(vs[1] * 2);
 
-  Phase ph[2];
-  const int n_phases = phases_for(r, default_hp(H / Hkv), ph);
-  if (n_phases < 0)
+  Shape ph;
+  if (!shape_for(r, default_hp(H / Hkv), &ph))
     return fail(INTRA_ERR_UNSUPPORTED, "block scatter with an offset needs block %% 256 == 0 unless H / Hkv is even (block %% 128) or a multiple of 4 (block %% 64)");
-  PhaseDims dims[2];
-  for (int i = 0; i < n_phases; ++i) {
-    dims[i] = by_map<DimsOf>(ph[i].map, r, ph[i]);
-    if (dims[i].work_items <= 0 || dims[i].n_pairs <= 0)
-      return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 work items");
-  }
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  for (int i = 0; i < n_phases; ++i) {  // the launches write disjoint rows of o
-    const int grid = launch_grid(dims[i].work_items);
-    if (grid <= 0)
-      return fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
-    p.geom = ph[i].geom;
-    p.n_sets = dims[i].n_sets;
-    p.n_mblocks = dims[i].n_mblocks;
-    p.hgroups = dims[i].hgroups;
-    p.n_pairs = dims[i].n_pairs;
-    p.items_per_pair = dims[i].hgroups * dims[i].n_mblocks;
-    p.n_slots = dims[i].work_items / 8;
-    p.d_items_per_pair = make_fastdiv(p.items_per_pair);
-    p.d_nbh = make_fastdiv(B * Hkv);
-    p.d_hkv = make_fastdiv(Hkv);
-    p.d_hgroups = make_fastdiv(p.hgroups);
-    rc = by_map<LaunchMap>(ph[i].map, p, ph[i].hp, ph[i].nw, grid, st);
-    if (rc) return rc;
-  }
-  return INTRA_OK;
+  const LaunchDims dims = by_map<DimsOf>(ph.map, r, ph);
+  if (dims.work_items <= 0 || dims.n_pairs <= 0)
+    return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 work items");
+  const int grid = launch_grid(dims.work_items);
+  if (grid <= 0)
+    return fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
+  p.geom = ph.geom;
+  p.n_sets = dims.n_sets;
+  p.n_mblocks = dims.n_mblocks;
+  p.hgroups = dims.hgroups;
+  p.n_pairs = dims.n_pairs;
+  p.items_per_pair = dims.hgroups * dims.n_mblocks;
+  p.n_slots = dims.work_items / 8;
+  p.d_items_per_pair = make_fastdiv(p.items_per_pair);
+  p.d_nbh = make_fastdiv(B * Hkv);
+  p.d_hkv = make_fastdiv(Hkv);
+  p.d_hgroups = make_fastdiv(p.hgroups);
+  return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, grid, static_cast<hipStream_t>(stream));
 }
 
 int model_mask(const Request& r, int heads_per_block, int waves, uint8_t* count) {
   const int hp = heads_per_block > 0 ? heads_per_block : 1;
   if ((hp != 1 && hp != 2 && hp != 4) || (waves > 0 && waves != 8))
     return fail(INTRA_ERR_INVALID, "no kernel for heads_per_block=%d, waves=%d", hp, waves);
-  Phase ph[2];
-  const int n_phases = phases_for(r, hp, ph);
-  if (n_phases < 0) return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
-  for (int i = 0; i < n_phases; ++i) by_map<ModelWalk>(ph[i].map, ph[i].geom, ph[i].hp, ph[i].nw, count);
+  Shape ph;
+  if (!shape_for(r, hp, &ph))
+    return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
+  by_map<ModelWalk>(ph.map, ph.geom, ph.hp, ph.nw, count);
   return INTRA_OK;
 }
 
