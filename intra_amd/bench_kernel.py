@@ -2,7 +2,9 @@
 
 Same protocol and CLI as the reference's benchmarks/bench_kernel.py:23-34,91-111 (median of
 --iters event-timed calls after --warmup calls; `llm` and `image` modes), with the rows extended
-by effective TFLOP/s (unmasked pairs only) and the fraction of the bf16 dense MFMA peak.
+by effective TFLOP/s (unmasked pairs only) and the fraction of the bf16 dense MFMA peak.  The rows
+keep the reference's keys with the latency in ms as value (benchmarks/results/*.json); the
+additions are `<key>_tflops`, `<key>_pct_peak` and the `*_run` stacks.
 
     python -m intra_amd.bench_kernel llm   --seqlens 4096,8192,16384,32768,65536
     python -m intra_amd.bench_kernel image
@@ -61,9 +63,13 @@ def qkv(B, S, H, Hkv, seed=0):
     return mk(H), mk(Hkv), mk(Hkv)
 
 
-def entry(ms, npairs, B, H):
+def put(row, key, ms, npairs, B, H):
+    """row[key] is the latency in ms, as in the reference's result files; the effective TFLOP/s
+    (unmasked pairs only) and the fraction of the bf16 MFMA peak go beside it."""
     tf = 4 * 128 * npairs * H * B / (ms * 1e-3) / 1e12
-    return {"ms": round(ms, 4), "tflops_eff": round(tf, 1), "pct_peak": round(100 * tf / PEAK_BF16_TFLOPS, 1)}
+    row[key] = round(ms, 4)
+    row[key + "_tflops"] = round(tf, 1)
+    row[key + "_pct_peak"] = round(100 * tf / PEAK_BF16_TFLOPS, 1)
 
 
 @torch.no_grad()
@@ -75,18 +81,20 @@ def bench_llm(args):
         r = {"seqlen": S}
         if args.dense:
             ms = median_ms(lambda: dense_sdpa(q, k, v, True), args.warmup, args.iters)
-            r["dense"] = entry(ms, S * (S + 1) // 2, B, H)
+            put(r, "dense", ms, S * (S + 1) // 2, B, H)
         for G in args.groups:
             ms = median_ms(lambda: intra_llm_attn(q, k, v, "scatter", group_num=G), args.warmup, args.iters)
-            r[f"scatter_g{G}"] = entry(ms, pairs(0, 0, B, S, H, Hkv, G, 576), B, H)
+            put(r, f"scatter_g{G}", ms, pairs(0, 0, B, S, H, Hkv, G, 576), B, H)
         if S % 64 == 0:
             ms = median_ms(lambda: intra_llm_attn(q, k, v, "gather1", group_num=8), args.warmup, args.iters)
-            r["gather1_g8"] = entry(ms, pairs(0, 1, B, S, H, Hkv, 8, 576), B, H)
+            put(r, "gather1_g8", ms, pairs(0, 1, B, S, H, Hkv, 8, 576), B, H)
         ms = median_ms(lambda: intra_llm_attn(q, k, v, "window", window=576), args.warmup, args.iters)
-        r["window576"] = entry(ms, pairs(0, 4, B, S, H, Hkv, 8, 576), B, H)
+        put(r, "window576", ms, pairs(0, 4, B, S, H, Hkv, 8, 576), B, H)
         if "scatter_g2" in r:
             # the reference's arithmetic for the 32-layer g2s4 schedule (bench_kernel.py:66-68) ...
-            r["g2s4_32layer_ms"] = round(4 * r["scatter_g2"]["ms"] + 28 * r["window576"]["ms"], 3)
+            r["g2s4_32layer"] = round(4 * r["scatter_g2"] + 28 * r["window576"], 3)
+            if "dense" in r:
+                r["dense_32layer"] = round(32 * r["dense"], 3)
             # ... and the same stack actually run back to back with fresh inputs per layer
             layers = [qkv(B, S, H, Hkv, seed=i) for i in range(4)]
 
@@ -97,7 +105,7 @@ def bench_llm(args):
                         intra_llm_attn(ql, kl, vl, "scatter", group_num=2)
                     else:
                         intra_llm_attn(ql, kl, vl, "window", window=576)
-            r["g2s4_32layer_run_ms"] = round(median_ms(stack, 2, max(3, args.iters // 10)), 3)
+            r["g2s4_32layer_run"] = round(median_ms(stack, 2, max(3, args.iters // 10)), 3)
         if args.model_patterns:
             # the layers the reference's model integration really runs in its g2s4 LLaMA setting
             # (experiments/llm/llama_intra.py:16-18): block Scatter with 2 groups of 256-token
@@ -105,9 +113,9 @@ def bench_llm(args):
             for off in (0, 1):
                 kw = dict(group_num=2, block=256, offset=off, n_sink=64)
                 ms = median_ms(lambda: intra_llm_attn(q, k, v, "block_scatter", **kw), args.warmup, args.iters)
-                r[f"block_scatter_g2_b256_off{off}_sink64"] = entry(ms, pairs_ex(8, B, S, H, Hkv, 2, 575, 256, off, 64), B, H)
+                put(r, f"block_scatter_g2_b256_off{off}_sink64", ms, pairs_ex(8, B, S, H, Hkv, 2, 575, 256, off, 64), B, H)
             ms = median_ms(lambda: intra_llm_attn(q, k, v, "window_sink", window=575, n_sink=64), args.warmup, args.iters)
-            r["window575_sink64"] = entry(ms, pairs_ex(9, B, S, H, Hkv, 2, 575, 256, 0, 64), B, H)
+            put(r, "window575_sink64", ms, pairs_ex(9, B, S, H, Hkv, 2, 575, 256, 0, 64), B, H)
             layers = [qkv(B, S, H, Hkv, seed=i) for i in range(4)]
 
             def model_stack():
@@ -117,7 +125,7 @@ def bench_llm(args):
                         intra_llm_attn(ql, kl, vl, "block_scatter", group_num=2, block=256, offset=(i // 8) % 2, n_sink=64)
                     else:
                         intra_llm_attn(ql, kl, vl, "window_sink", window=575, n_sink=64)
-            r["g2s4_model_32layer_run_ms"] = round(median_ms(model_stack, 2, max(3, args.iters // 10)), 3)
+            r["g2s4_model_32layer_run"] = round(median_ms(model_stack, 2, max(3, args.iters // 10)), 3)
         rows.append(r)
         print(json.dumps(r), flush=True)
     return rows
@@ -132,11 +140,11 @@ def bench_image(args):
         q, k, v = qkv(B, S, H, H)
         r = {"width": width, "seqlen": S}
         if args.dense:
-            r["dense"] = entry(median_ms(lambda: dense_sdpa(q, k, v, False), args.warmup, args.iters), S * S, B, H)
+            put(r, "dense", median_ms(lambda: dense_sdpa(q, k, v, False), args.warmup, args.iters), S * S, B, H)
         for pattern, pid in (("scatter", 0), ("gather0", 4)):
             ms = median_ms(lambda: intra_image_attn(q, k, v, pattern, width), args.warmup, args.iters)
-            r[pattern] = entry(ms, pairs(1, pid, B, S, H, H, width, TEXT_LEN), B, H)
-        r["interleaved_mean_ms"] = round((r["scatter"]["ms"] + r["gather0"]["ms"]) / 2, 4)
+            put(r, pattern, ms, pairs(1, pid, B, S, H, H, width, TEXT_LEN), B, H)
+        r["interleaved_mean"] = round((r["scatter"] + r["gather0"]) / 2, 4)  # layers alternate the two patterns
         rows.append(r)
         print(json.dumps(r), flush=True)
     return rows
