@@ -252,18 +252,36 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   }
   // Q^T fragments: lane holds query l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
   bf16x8 qf[8];
-  // this lane's query row of a work item (clamped to the last row of the row block)
-  auto q_row = [&](const Where& w) {
-    const MAP map(p.geom, w.set, w.mblk * POS);
-    const int t1 = im_min(w.mblk * POS + POS, map.nq()) - 1;
-    const int tq = im_min(w.mblk * POS + (wave / HP) * 32 + l32, t1);
-    const int hq = w.kvh * p.ratio + w.hg * HP + wave % HP;
-    return w.batch * p.q_bs + (int64_t)map.qpos(tq) * p.q_rs + hq * p.q_hs + h32 * 8;
+  // Q is fetched, and O stored, 64 contiguous bytes per row and instruction instead of 32: the two
+  // lanes of neighbouring queries 2a, 2a+1 (and their upper-half twins) together cover chunks
+  // 4m..4m+3 of row 2a in access 2m and of row 2a+1 in access 2m+1, lane (e = query parity, h)
+  // taking chunk 4m + 2e + h.  A lane then holds its own chunks 2ks + h only for ks = e (mod 2);
+  // the others sit in its neighbour and are swapped in with one quad permute per dword
+  // (pair_exchange, its own inverse).  Rows past the end of the row block are clamped to its
+  // last row.
+  const int qpar = l32 & 1;
+  auto pair_exchange = [&](u32x4 (&r)[8]) {
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        const uint32_t x0 = r[2 * m][d], x1 = r[2 * m + 1][d];
+        const uint32_t got = (uint32_t)__builtin_amdgcn_mov_dpp((int)(qpar ? x0 : x1), 0xB1, 0xF, 0xF, true);  // lane ^ 1
+        r[2 * m][d] = qpar ? got : x0;
+        r[2 * m + 1][d] = qpar ? x1 : got;
+      }
   };
   auto load_q = [&](const Where& w) {
-    const uint16_t* qrow = p.q + q_row(w);
+    const MAP map(p.geom, w.set, w.mblk * POS);
+    const int t1 = im_min(w.mblk * POS + POS, map.nq()) - 1;
+    const int r0 = w.mblk * POS + (wave / HP) * 32 + (l32 & ~1);
+    const int hq = w.kvh * p.ratio + w.hg * HP + wave % HP;
+    const int64_t head = w.batch * p.q_bs + hq * p.q_hs + (2 * qpar + h32) * 8;
+    const uint16_t* row_a = p.q + (head + (int64_t)map.qpos(im_min(r0, t1)) * p.q_rs);
+    const uint16_t* row_b = p.q + (head + (int64_t)map.qpos(im_min(r0 + 1, t1)) * p.q_rs);
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qrow + ks * 16);
+    for (int i = 0; i < 8; ++i)
+      qf[i] = *reinterpret_cast<const bf16x8*>(((i & 1) ? row_b : row_a) + 32 * (i >> 1));
   };
 
   // Ring slots (byte offsets into the K ring; the V ring uses the same offsets behind VBASE) of
@@ -314,14 +332,23 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
 
   const int hq = kvh * p.ratio + hg * HP + hw;
   const int64_t qpos = map.qpos(tq);
+  // the two rows this lane stores parts of (see load_q), and whether they exist
+  const int ra = wq0 + (l32 & ~1);
+  const int64_t opos_a = map.qpos(im_min(ra, t1)), opos_b = map.qpos(im_min(ra + 1, t1));
+  const bool valid_a = ra <= t1, valid_b = ra + 1 <= t1;
   // Pin the arrival of Q here: the empty asm uses and redefines the fragments, so the compiler waits
   // for their loads at this point (where the wait is needed anyway) and not, with a counter value
   // that also covers the tile requests in flight, in front of every MFMA that reads them.
+  {
+    u32x4 raw[8];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) {
-    u32x4 t = __builtin_bit_cast(u32x4, qf[ks]);
-    asm volatile("" : "+v"(t));
-    qf[ks] = __builtin_bit_cast(bf16x8, t);
+    for (int ks = 0; ks < 8; ++ks) {
+      raw[ks] = __builtin_bit_cast(u32x4, qf[ks]);
+      asm volatile("" : "+v"(raw[ks]));
+    }
+    pair_exchange(raw);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = __builtin_bit_cast(bf16x8, raw[ks]);
   }
   if (p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
 #pragma unroll
@@ -544,8 +571,9 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     p.lse[batch * p.lse_bs + hq * p.lse_hs + qpos * p.lse_ts] = (mref + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   // Lane l and lane l+32 hold the same query: per 16 head dims the lower lane has dims 0-3 and
   // 8-11, the upper one 4-7 and 12-15.  One permlane32 swap per register pair turns that into
-  // dims 0-7 / 8-15, so each lane writes 16 contiguous bytes.
-  uint16_t* orow = p.o + batch * p.o_bs + qpos * p.o_rs + hq * p.o_hs + 8 * h32;
+  // dims 0-7 / 8-15, i.e. 16-byte chunk 2*ks + h of the row for ks = 2*db + g2; pair_exchange
+  // then regroups the chunks so that four lanes store 64 contiguous bytes of one row.
+  u32x4 pk[8];
 #pragma unroll
   for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -561,11 +589,17 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
         }
       auto r0 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
       auto r1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
-      if (row_valid) {
-        u32x4 pk = {r0[0], r1[0], r0[1], r1[1]};
-        *reinterpret_cast<u32x4*>(orow + 32 * db + 16 * g2) = pk;
-      }
+      pk[2 * db + g2] = u32x4{r0[0], r1[0], r0[1], r1[1]};
     }
+  pair_exchange(pk);
+  const int64_t ohead = batch * p.o_bs + hq * p.o_hs + (2 * qpar + h32) * 8;
+  uint16_t* orow_a = p.o + (ohead + opos_a * p.o_rs);
+  uint16_t* orow_b = p.o + (ohead + opos_b * p.o_rs);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    if ((i & 1) ? valid_b : valid_a)
+      *reinterpret_cast<u32x4*>(((i & 1) ? orow_b : orow_a) + 32 * (i >> 1)) = pk[i];
+  }
   }
   if (!more) break;
   cw = nw;
