@@ -357,3 +357,33 @@ def test_new_pair_counts_match_masks():
     rows = torch.tensor([0, 5, 99])
     assert torch.equal(oracle.mask_rows("llm/window_sink", 100, rows=rows, window=10, n_sink=3),
                        masks.llm_window_sink_mask(100, 10, 3)[rows])
+
+
+def test_reference_known_answers():
+    """tests/golden/reference_known_answers.json: every point, count and density the reference
+    asserts or prints about its own masks."""
+    import json
+    import os
+    path = os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")
+    data = json.load(open(path))
+    for entry in data["masks"]:
+        m = oracle.mask_rows(entry["kind"], entry["S"], **entry["args"])
+        for q, k in entry.get("true", []):
+            assert bool(m[q, k]), (entry["source"], q, k)
+        for q, k in entry.get("false", []):
+            assert not bool(m[q, k]), (entry["source"], q, k)
+        if "all_true_columns_below" in entry:
+            assert bool(m[:, :entry["all_true_columns_below"]].all())
+        if "grid_keys_per_grid_row" in entry:
+            T = oracle.TEXT_LEN
+            assert bool(m[T:, T:].sum(1).eq(entry["grid_keys_per_grid_row"]).all())
+        if "density_percent" in entry:
+            assert round(100.0 * m.float().mean().item(), 2) == entry["density_percent"]
+    for entry in data["brute_force"]:
+        S, G = entry["S"], entry["args"]["group_num"]
+        m = oracle.mask_rows(entry["kind"], S, **entry["args"])
+        for q in range(S):
+            for k in range(S):
+                assert bool(m[q, k]) == bool(eval(entry["rule"], {"q": q, "k": k, "G": G}))
+    for entry in data["pairs"]:
+        assert pairs.pairs_per_head(entry["kind"], entry["S"], **entry["args"]) == entry["pairs_per_head"]
