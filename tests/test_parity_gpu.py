@@ -376,3 +376,25 @@ def test_random_llm_shapes(case):
     check(out, q, k, v, f"llm/{kind}", scale=scale, rtol=2.0 ** -7, **kw)
     ref = oracle.masked_lse_rows(q, k, oracle.mask_rows(f"llm/{kind}", S, device=DEV, **kw), softmax_scale=scale)
     assert (lse - ref).abs().max().item() <= LSE_ATOL
+
+
+@pytest.mark.parametrize("width,text_len,H,Hkv", [(24, 72, 4, 4), (40, 8, 8, 2), (16, 200, 2, 1), (32, 96, 4, 1)])
+@pytest.mark.parametrize("pattern,pid", [("scatter", 0), ("gather0", 4)])
+def test_image_other_text_lengths_through_the_c_abi(width, text_len, H, Hkv, pattern, pid):
+    """The Python entry point fixes 512 text tokens like the reference; the C ABI takes any multiple
+    of 8, including prefixes that end inside a 32-key block."""
+    from intra_amd import _lib
+    lib = _lib.load()
+    S = text_len + width * width
+    q, k, v = make_qkv(2, S, H, Hkv, seed=61)
+    out = torch.empty_like(q)
+    lse = torch.empty(2, H, S, dtype=torch.float32, device=DEV)
+    rc = lib.intra_image_fwd_lse(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), 2, S, H, Hkv,
+                                 _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                                 pid, width, text_len, 128 ** -0.5,
+                                 torch.cuda.current_stream().cuda_stream, lse.data_ptr(), _lib.strides3(lse))
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    check(out, q, k, v, f"image/{pattern}", width=width, text_len=text_len)
+    mask = oracle.mask_rows(f"image/{pattern}", S, device=DEV, width=width, text_len=text_len)
+    assert (lse - oracle.masked_lse_rows(q, k, mask)).abs().max().item() <= LSE_ATOL
