@@ -43,3 +43,35 @@ def test_rejects_non_cuda_bf16_128(make):
         intra_amd.intra_llm_attn(q, k, v)
     with pytest.raises(ValueError, match="CUDA bfloat16 tensors with head_dim 128"):
         intra_amd.intra_image_attn(q, k, v)
+
+
+def test_missing_library_fails_loudly_and_nothing_falls_back(tmp_path):
+    """Without the native library the package still imports (as the reference's does), but every
+    call raises ImportError: there is no CPU or PyTorch fallback path."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("import torch, intra_amd\n"
+            "q = torch.zeros(1, 64, 4, 128, dtype=torch.bfloat16)\n"
+            "for fn in (intra_amd.intra_llm_attn, intra_amd.intra_image_attn):\n"
+            "    try:\n"
+            "        fn(q, q, q)\n"
+            "    except ImportError as e:\n"
+            "        assert 'not built' in str(e)\n"
+            "    else:\n"
+            "        raise SystemExit('call succeeded without the library')\n"
+            "print('ok')\n")
+    env = dict(os.environ, INTRA_HIP_LIB=str(tmp_path / "nowhere.so"), PYTHONPATH=root)
+    res = subprocess.run([sys.executable, "-c", code], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert res.returncode == 0 and res.stdout.strip().endswith("ok"), res.stdout
+
+
+def test_product_never_imports_the_oracle():
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for pkg in ("intra_amd", "intra_attn"):
+        for name in os.listdir(os.path.join(root, pkg)):
+            if name.endswith(".py"):
+                text = open(os.path.join(root, pkg, name)).read()
+                assert "import oracle" not in text and "from oracle" not in text, f"{pkg}/{name}"
