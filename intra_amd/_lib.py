@@ -1,5 +1,6 @@
 """ctypes binding of libintra_hip.so (declared in include/intra_hip.h)."""
 import ctypes
+import functools
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -64,6 +65,12 @@ def last_error():
     return load().intra_last_error().decode()
 
 
+@functools.lru_cache(maxsize=256)
+def _strides_array(s0, s1, s2):
+    return _i64x3(s0, s1, s2)
+
+
 def strides3(x):
-    """(batch, token, head) element strides of a (B, S, H, D) tensor as a C array."""
-    return _i64x3(x.stride(0), x.stride(1), x.stride(2))
+    """The first three element strides of a tensor ((batch, token, head) of a (B, S, H, D) tensor)
+    as a C array; the arrays are read-only for the library and cached."""
+    return _strides_array(x.stride(0), x.stride(1), x.stride(2))

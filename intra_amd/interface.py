@@ -7,6 +7,8 @@ divide the query heads.  Pattern names, arguments, defaults and exception types 
 reference's.  The work is done by libintra_hip.so through its C ABI (include/intra_hip.h); there
 is no fallback path, a missing library is an ImportError.
 """
+import contextlib
+
 import torch
 
 from . import _lib
@@ -46,6 +48,14 @@ def _scale(q, softmax_scale):
     return q.shape[-1] ** -0.5 if softmax_scale is None else softmax_scale
 
 
+def _stream_on(device):
+    """(context that makes `device` current, handle of its current stream).  Switching devices is
+    only paid for when the tensors live on another GPU than the current one."""
+    if device.index == torch.cuda.current_device():
+        return contextlib.nullcontext(), torch.cuda.current_stream().cuda_stream
+    return torch.cuda.device(device), torch.cuda.current_stream(device).cuda_stream
+
+
 def _launch(fn, fn_lse, q, k, v, pattern_id, arg0, arg1, scale, return_lse=False):
     out = torch.empty_like(q)
     if not _aligned(out):
@@ -55,8 +65,8 @@ def _launch(fn, fn_lse, q, k, v, pattern_id, arg0, arg1, scale, return_lse=False
             _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
             pattern_id, arg0, arg1, float(scale)]
     lse = torch.empty(B, H, S, dtype=torch.float32, device=q.device) if return_lse else None
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream(q.device).cuda_stream
+    guard, stream = _stream_on(q.device)
+    with guard:
         if return_lse:
             rc = fn_lse(*args, stream, lse.data_ptr(), _lib.strides3(lse))
         else:
@@ -72,8 +82,8 @@ def _launch_ex(q, k, v, pattern_id, group_num, window, block, offset, n_sink, sc
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     B, S, H, _ = q.shape
     lse = torch.empty(B, H, S, dtype=torch.float32, device=q.device) if return_lse else None
-    with torch.cuda.device(q.device):
-        stream = torch.cuda.current_stream(q.device).cuda_stream
+    guard, stream = _stream_on(q.device)
+    with guard:
         rc = _C.intra_llm_fwd_ex(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
                                  _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
                                  pattern_id, group_num, window, block, offset, n_sink, float(scale), stream,
