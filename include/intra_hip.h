@@ -103,6 +103,29 @@ const char* intra_last_error(void);
 /* Library version, major*10000 + minor*100 + patch. */
 int intra_version(void);
 
+/* Backward pass of intra_llm_fwd / intra_llm_fwd_ex: gradients of the inputs given the gradient
+ * `dout` of the output.  The reference ships no backward kernels (README.md lists them as missing;
+ * its training experiments differentiate masked SDPA / FlexAttention instead,
+ * experiments/llm/llama_intra.py:26); this entry point has no counterpart there and is what an
+ * autograd wrapper of intra_llm_attn needs.
+ *   o, lse:    output and log-sum-exp of the forward call with the same arguments
+ *   dout:      gradient of o, bf16, shaped like q
+ *   dq/dk/dv:  results, bf16, shaped like q / k / v (every element is written)
+ *   workspace: B * H * S floats of device memory owned by the caller (holds rowsum(dout * o));
+ *              contents on entry do not matter
+ * Patterns: 0, 1, 4 and INTRA_LLM_BLOCK_SCATTER with offset = 0 and n_sink = 0; others return
+ * INTRA_ERR_UNSUPPORTED.  Three launches on hip_stream (dq, then dk, then dv); nothing is
+ * allocated.  Accuracy: weights are rounded to bf16 before the second product, as in the forward
+ * pass, accumulation is fp32. */
+int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse,
+                  const void* dout, void* dq, void* dk, void* dv, float* workspace, int B, int S,
+                  int H, int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                  const int64_t v_strides[3], const int64_t o_strides[3],
+                  const int64_t dout_strides[3], const int64_t dq_strides[3],
+                  const int64_t dk_strides[3], const int64_t dv_strides[3],
+                  const int64_t lse_strides[3], int pattern, int group_num, int window, int block,
+                  int offset, int n_sink, float softmax_scale, void* hip_stream);
+
 /* ------------------------------------------------------------------ host-only helpers (no GPU)
  * How a call would be launched; mirrors the grid / per-set length derivation of the reference
  * launchers (csrc/flash_attn/src/flash_fwd_launch_template.h:401-565, flash_api.cpp:408-411,

@@ -9,6 +9,7 @@
 
 #include "../../include/intra_hip.h"
 #include "intra_kernel.hip.h"
+#include "intra_bwd_kernel.hip.h"
 
 namespace {
 
@@ -383,6 +384,104 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, grid, static_cast<hipStream_t>(stream));
 }
 
+
+// ------------------------------------------------------------------------------------ backward
+template <class MAP, int MODE, int HP>
+int launch_bwd(const intra::BParams& p, int64_t grid, hipStream_t stream) {
+  if (grid <= 0 || grid > 0x7fffffff) return fail(INTRA_ERR_UNSUPPORTED, "backward needs more than 2^31 workgroups");
+  hipLaunchKernelGGL((intra::intra_bwd_kernel<MAP, MODE, HP>), dim3((unsigned)grid), dim3(512), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+  return INTRA_OK;
+}
+
+template <class MAP>
+int run_bwd_map(intra::BParams p, int hp, const Request& r, hipStream_t stream) {
+  const int64_t pairs = (int64_t)MAP::num_sets(p.geom) * r.B * r.Hkv;
+  const int max_rows = MAP::max_nq(p.geom);  // these maps number queries and keys alike: nq == nk
+  // dQ: row blocks of 256 / hp queries of hp heads; writes D = rowsum(dO o O) for the dK launch
+  p.hgroups = (r.H / r.Hkv) / hp;
+  p.n_rblocks = (max_rows + 256 / hp - 1) / (256 / hp);
+  int rc;
+  switch (hp) {
+    case 4: rc = launch_bwd<MAP, intra::BWD_DQ, 4>(p, pairs * p.n_rblocks * p.hgroups, stream); break;
+    case 2: rc = launch_bwd<MAP, intra::BWD_DQ, 2>(p, pairs * p.n_rblocks * p.hgroups, stream); break;
+    default: rc = launch_bwd<MAP, intra::BWD_DQ, 1>(p, pairs * p.n_rblocks * p.hgroups, stream); break;
+  }
+  if (rc) return rc;
+  // dK, dV: row blocks of 256 keys of one kv head, all query heads of its group streamed past
+  p.hgroups = 1;
+  p.n_rblocks = (max_rows + 255) / 256;
+  if ((rc = launch_bwd<MAP, intra::BWD_DK, 1>(p, pairs * p.n_rblocks, stream))) return rc;
+  return launch_bwd<MAP, intra::BWD_DV, 1>(p, pairs * p.n_rblocks, stream);
+}
+
+int run_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
+            void* dq, void* dk, void* dv, float* dsum, int B, int S, int H, int Hkv, const int64_t* qs,
+            const int64_t* ks, const int64_t* vs, const int64_t* os, const int64_t* dos, const int64_t* dqs,
+            const int64_t* dks, const int64_t* dvs, const int64_t* ls, int pattern, int group_num, int window,
+            int block, int offset, int n_sink, float scale, void* stream) {
+  g_err[0] = 0;
+  Request r;
+  int rc = make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true);
+  if (rc) return rc;
+  if (r.kind == KIND_LLM_WINDOW_SINK || (r.kind == KIND_LLM_BLOCK_SCATTER && (offset != 0 || n_sink != 0)))
+    return fail(INTRA_ERR_UNSUPPORTED,
+                "backward: dK / dV are built for scatter, gather1, window and block scatter without offset and sinks");
+  const void* ins[] = {q, k, v, o, dout, dq, dk, dv};
+  for (const void* ptr : ins) {
+    if (!ptr) return fail(INTRA_ERR_INVALID, "q, k, v, o, dout, dq, dk and dv must be non-null device pointers");
+    if (!aligned16(ptr)) return fail(INTRA_ERR_INVALID, "q, k, v, o, dout, dq, dk and dv must be 16-byte aligned");
+  }
+  if (!lse || !dsum || (reinterpret_cast<uintptr_t>(lse) & 3) || (reinterpret_cast<uintptr_t>(dsum) & 3))
+    return fail(INTRA_ERR_INVALID, "lse and the workspace must be non-null, 4-byte aligned device pointers");
+  if ((rc = check_strides("q", qs, B, S, H)) || (rc = check_strides("k", ks, B, S, Hkv)) ||
+      (rc = check_strides("v", vs, B, S, Hkv)) || (rc = check_strides("o", os, B, S, H)) ||
+      (rc = check_strides("dout", dos, B, S, H)) || (rc = check_strides("odq", dqs, B, S, H)) ||
+      (rc = check_strides("odk", dks, B, S, Hkv)) || (rc = check_strides("odv", dvs, B, S, Hkv)))
+    return rc;
+  if (!ls) return fail(INTRA_ERR_INVALID, "lse strides pointer is null");
+  if (!isfinite(scale)) return fail(INTRA_ERR_INVALID, "softmax_scale must be finite");
+  const int64_t* all[] = {qs, ks, vs, dos};
+  for (const int64_t* st : all)
+    if (st[1] >= ((int64_t)1 << 31)) return fail(INTRA_ERR_UNSUPPORTED, "token strides must stay below 2^31 elements");
+
+  intra::BParams p;
+  p.q = static_cast<const uint16_t*>(q);
+  p.k = static_cast<const uint16_t*>(k);
+  p.v = static_cast<const uint16_t*>(v);
+  p.o = static_cast<const uint16_t*>(o);
+  p.dout = static_cast<const uint16_t*>(dout);
+  p.lse = lse;
+  p.dsum = dsum;
+  p.dq = static_cast<uint16_t*>(dq);
+  p.dk = static_cast<uint16_t*>(dk);
+  p.dv = static_cast<uint16_t*>(dv);
+  p.q_bs = qs[0]; p.q_rs = qs[1]; p.q_hs = qs[2];
+  p.k_bs = ks[0]; p.k_rs = ks[1]; p.k_hs = ks[2];
+  p.v_bs = vs[0]; p.v_rs = vs[1]; p.v_hs = vs[2];
+  p.o_bs = os[0]; p.o_rs = os[1]; p.o_hs = os[2];
+  p.do_bs = dos[0]; p.do_rs = dos[1]; p.do_hs = dos[2];
+  p.dq_bs = dqs[0]; p.dq_rs = dqs[1]; p.dq_hs = dqs[2];
+  p.dk_bs = dks[0]; p.dk_rs = dks[1]; p.dk_hs = dks[2];
+  p.dv_bs = dvs[0]; p.dv_rs = dvs[1]; p.dv_hs = dvs[2];
+  p.lse_bs = ls[0]; p.lse_hs = ls[1]; p.lse_ts = ls[2];
+  p.ds_bs = (int64_t)H * S; p.ds_hs = S;
+  p.B = B; p.H = H; p.Hkv = Hkv; p.ratio = H / Hkv;
+  p.scale = scale;
+  p.scale_log2 = scale * 1.4426950408889634f;
+  Shape sh;
+  if (!shape_for(r, default_hp(H / Hkv), &sh)) return fail(INTRA_ERR_UNSUPPORTED, "no kernel shape for this request");
+  p.geom = sh.geom;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  switch (sh.map) {
+    case MAP_LLM_SCATTER: return run_bwd_map<MapLlmScatter>(p, sh.hp, r, st);
+    case MAP_LLM_GATHER1: return run_bwd_map<MapLlmGather1>(p, sh.hp, r, st);
+    case MAP_LLM_WINDOW: return run_bwd_map<MapLlmWindow>(p, sh.hp, r, st);
+    default: return run_bwd_map<MapLlmBlockScatter>(p, sh.hp, r, st);
+  }
+}
+
 int model_mask(const Request& r, int heads_per_block, int waves, uint8_t* count) {
   const int hp = heads_per_block > 0 ? heads_per_block : 1;
   if ((hp != 1 && hp != 2 && hp != 4) || (waves > 0 && waves != 8))
@@ -430,6 +529,18 @@ int intra_image_fwd_lse(const void* q, const void* k, const void* v, void* o, in
                         const int64_t lse_strides[3]) {
   return run(1, q, k, v, o, B, S, H, Hkv, q_strides, k_strides, v_strides, o_strides, pattern,
              width, text_len, softmax_scale, hip_stream, lse, lse_strides, true);
+}
+
+int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
+                  void* dq, void* dk, void* dv, float* workspace, int B, int S, int H, int Hkv,
+                  const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                  const int64_t o_strides[3], const int64_t dout_strides[3], const int64_t dq_strides[3],
+                  const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[3],
+                  int pattern, int group_num, int window, int block, int offset, int n_sink,
+                  float softmax_scale, void* hip_stream) {
+  return run_bwd(q, k, v, o, lse, dout, dq, dk, dv, workspace, B, S, H, Hkv, q_strides, k_strides, v_strides,
+                 o_strides, dout_strides, dq_strides, dk_strides, dv_strides, lse_strides, pattern, group_num,
+                 window, block, offset, n_sink, softmax_scale, hip_stream);
 }
 
 const char* intra_last_error(void) { return g_err; }

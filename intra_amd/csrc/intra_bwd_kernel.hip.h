@@ -1,0 +1,337 @@
+// Backward kernels of the sparse attention for gfx950 (MI355X): dQ for every pattern, dK / dV for
+// the patterns whose sets number queries and keys alike (LLM Scatter, Gather 1, 64-aligned window,
+// block Scatter without offset and sinks).
+//
+// The reference has no backward kernels (its README names them as missing; training there runs
+// through masked SDPA / FlexAttention, experiments/llm/llama_intra.py:26).  The math is the usual
+//   P = exp(scale * S - lse),  dV = P^T dO,  dP = dO V^T,  dS = P o (dP - D),  D_i = dO_i . O_i,
+//   dQ = scale * dS K,  dK = scale * dS^T Q.
+//
+// One template serves the three results.  A workgroup owns 256 / HP "rows" (queries for dQ, keys
+// for dK and dV; 32 per wavefront, held as MFMA B operands in registers like Q in the forward
+// kernel) and streams the "columns" that see them through LDS in tiles of 64 (K and V rows for
+// dQ, Q and dO rows of every query head of the group for dK / dV), double buffered.  Per 32
+// columns a wavefront forms the scores S^T = C1 R1^T and dP^T = C2 R2^T, turns them into the
+// weights (P or dS), packed to bf16 straight from the accumulators, and adds X^T W^T to its
+// accumulators, X being the K, Q or dO tile read with transposing LDS reads - the data flow of
+// the forward kernel without the online softmax.  Which columns a row meets follows from the same
+// index maps; for dK / dV the query range of a key is found by bisection on the maps' monotone
+// bounds, so no pattern needs inverse formulas.
+#pragma once
+#include "intra_kernel.hip.h"
+
+namespace intra {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+enum BwdMode : int { BWD_DQ = 0, BWD_DK = 1, BWD_DV = 2 };
+
+struct BParams {
+  const uint16_t *q, *k, *v, *o, *dout;  // bf16 (B, S, heads, 128)
+  const float* lse;                      // (B, H, S): ln sum exp(scale * q.k) from the forward pass
+  float* dsum;                           // (B, H, S) workspace: D = rowsum(dO o O), written by dQ, read by dK
+  uint16_t *dq, *dk, *dv;
+  // element strides: batch, row (token), head
+  int64_t q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs, o_hs, do_bs, do_rs, do_hs;
+  int64_t dq_bs, dq_rs, dq_hs, dk_bs, dk_rs, dk_hs, dv_bs, dv_rs, dv_hs;
+  int64_t lse_bs, lse_hs, lse_ts, ds_bs, ds_hs;  // dsum is contiguous over tokens
+  int B, H, Hkv, ratio;
+  IntraGeom geom;
+  float scale;       // softmax scale
+  float scale_log2;  // scale * log2(e)
+  int n_rblocks;     // row blocks per set
+  int hgroups;       // ratio / HP (dQ only)
+};
+
+constexpr int BWD_SLOT = 2 * TILE_BYTES + 512;  // two tiles and 2 x 64 column scalars
+constexpr int BWD_LDS_BYTES = 2 * BWD_SLOT;
+
+template <class MAP, int MODE, int HP>
+__global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
+  constexpr int NW = 8;
+  constexpr bool ROWS_ARE_QUERIES = MODE == BWD_DQ;
+  constexpr int POS = ROWS_ARE_QUERIES ? NW * 32 / HP : NW * 32;  // rows per row block (of one head)
+  static_assert(ROWS_ARE_QUERIES || !MAP::kHasPrefix, "dK / dV need a per-set key numbering without prefix");
+
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[BWD_LDS_BYTES];
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int h32 = lane >> 5;
+  const int l32 = lane & 31;
+
+  // ---------------------------------------------------------------- work item
+  int item = blockIdx.x;
+  int hg = 0;
+  if (ROWS_ARE_QUERIES) {
+    hg = item % p.hgroups;
+    item /= p.hgroups;
+  }
+  const int rblk = item % p.n_rblocks;
+  const int pair = item / p.n_rblocks;
+  const int nbh = p.B * p.Hkv;
+  const int set = pair / nbh;
+  const int bh = pair % nbh;
+  const int batch = bh / p.Hkv;
+  const int kvh = bh % p.Hkv;
+
+  const int r0 = rblk * POS;
+  const MAP map(p.geom, set, ROWS_ARE_QUERIES ? r0 : 0);
+  const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
+  const int n_rows = ROWS_ARE_QUERIES ? nq : nk;
+  const int n_cols = ROWS_ARE_QUERIES ? nk : nq;
+  if (r0 >= n_rows) return;
+  const int r1 = im_min(r0 + POS, n_rows) - 1;
+
+  // Columns a row meets: [col_lo(r), col_hi(r)] (plus the prefix below kpre for maps that have one).
+  // For key rows the bounds are the first query whose upper key bound reaches the key and the last
+  // one whose lower key bound does not exceed it; both are monotone in the key.
+  auto col_lo = [&](int r) {
+    if (ROWS_ARE_QUERIES) return map.klo(r);
+    int lo = 0, hi = nq;  // first tq with min(khi(tq), nk-1) >= r
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (im_min(map.khi(mid), nk - 1) >= r) hi = mid;
+      else lo = mid + 1;
+    }
+    return lo;
+  };
+  auto col_hi = [&](int r) {
+    if (ROWS_ARE_QUERIES) return im_min(map.khi(r), nk - 1);
+    int lo = -1, hi = nq - 1;  // last tq with klo(tq) <= r
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (map.klo(mid) <= r) lo = mid;
+      else hi = mid - 1;
+    }
+    return lo;
+  };
+
+  const int cb = (ROWS_ARE_QUERIES && MAP::kHasPrefix) ? 0 : col_lo(r0);  // first column of the row block
+  const int ce = col_hi(r1);                                             // last one
+  const int ntiles = ce >= cb ? (ce - cb + BN) / BN : 0;
+
+  // ---------------------------------------------------------------- this wavefront's rows
+  const int hw = ROWS_ARE_QUERIES ? wave % HP : 0;
+  const int wr0 = r0 + (ROWS_ARE_QUERIES ? wave / HP : wave) * 32;
+  const bool wave_active = wr0 <= r1;
+  const int wr_last = im_min(wr0 + 31, r1);
+  const bool row_valid = wr0 + l32 <= r1;
+  const int row = im_min(wr0 + l32, r1);
+  const int lo_l = col_lo(row), hi_l = col_hi(row);
+  WaveBounds wb;
+  wb.w_lo = __builtin_amdgcn_readfirstlane(col_lo(im_min(wr0, r1)));
+  wb.w_hi = __builtin_amdgcn_readfirstlane(col_hi(wr_last));
+  wb.f_lo = __builtin_amdgcn_readfirstlane(col_lo(wr_last));
+  wb.f_hi = __builtin_amdgcn_readfirstlane(col_hi(im_min(wr0, r1)));
+  const int64_t rpos = ROWS_ARE_QUERIES ? map.qpos(row) : map.kpos(row);
+  const int hq = kvh * p.ratio + hg * HP + hw;  // query head of a query row
+
+  // ---------------------------------------------------------------- row operands (MFMA B fragments)
+  // lane holds row l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
+  bf16x8 r1f[8], r2f[8];
+  float L2_row = 0.f, D_row = 0.f;
+  {
+    const uint16_t *a1, *a2;
+    if (ROWS_ARE_QUERIES) {
+      a1 = p.q + (batch * p.q_bs + rpos * p.q_rs + hq * p.q_hs + h32 * 8);
+      a2 = p.dout + (batch * p.do_bs + rpos * p.do_rs + hq * p.do_hs + h32 * 8);
+    } else {
+      a1 = p.k + (batch * p.k_bs + rpos * p.k_rs + kvh * p.k_hs + h32 * 8);
+      a2 = p.v + (batch * p.v_bs + rpos * p.v_rs + kvh * p.v_hs + h32 * 8);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      r1f[ks] = *reinterpret_cast<const bf16x8*>(a1 + ks * 16);
+      if (MODE != BWD_DV) r2f[ks] = *reinterpret_cast<const bf16x8*>(a2 + ks * 16);
+    }
+    if (ROWS_ARE_QUERIES) {
+      // D = dO . O of the row: this lane's 64 head dims, then the other half from lane ^ 32
+      const uint16_t* ao = p.o + (batch * p.o_bs + rpos * p.o_rs + hq * p.o_hs + h32 * 8);
+      float part = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 of = *reinterpret_cast<const bf16x8*>(ao + ks * 16);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) part += (float)r2f[ks][d] * (float)of[d];
+      }
+      D_row = lane_xor32_sum(part);
+      L2_row = p.lse[batch * p.lse_bs + hq * p.lse_hs + rpos * p.lse_ts] * 1.4426950408889634f;
+      if (row_valid && h32 == 0) p.dsum[batch * p.ds_bs + hq * p.ds_hs + rpos] = D_row;
+    }
+  }
+
+  // ---------------------------------------------------------------- LDS addressing (as in the forward kernel)
+  const int ld_row = lane >> 4;
+  const uint32_t ld_col = (((lane & 15) ^ (4 * ld_row)) << 4);
+  int kaddr[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks)
+    kaddr[ks] = (l32 >> 2) * GROUP_STRIDE + (l32 & 3) * 256 + (((2 * ks + h32) ^ (4 * (l32 & 3))) << 4);
+  int vaddr[4];
+  {
+    const int i16 = lane & 15, g2 = (lane >> 4) & 1, ri = i16 >> 2;
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+      vaddr[db] = h32 * GROUP_STRIDE + ri * 256 + (((4 * db + 2 * g2 + ((i16 & 3) >> 1)) ^ (4 * ri)) << 4) + 8 * (i16 & 1);
+  }
+  auto kread = [&](int off, int ks) { return *reinterpret_cast<const bf16x8*>(smem + off + kaddr[ks]); };
+  auto vread = [&](int off, int j) {
+    const int o2 = off + vaddr[j & 3] + (j >> 2) * 4 * GROUP_STRIDE;
+    bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(smem + o2));
+    bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (__attribute__((address_space(3))) bf16x4*)(smem + o2 + 2 * GROUP_STRIDE));
+    return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+
+  floatx16 acc[4];
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
+  const float c2 = p.scale_log2;
+
+  // ---------------------------------------------------------------- column streams
+  // dQ: one stream (the K / V rows of the kv head); dK, dV: one per query head of the group.
+  const int n_streams = ROWS_ARE_QUERIES ? 1 : p.ratio;
+  for (int sidx = 0; sidx < n_streams; ++sidx) {
+    const int hcol = kvh * p.ratio + sidx;  // query head of the columns (dK / dV)
+    const char *c1base, *c2base;
+    uint32_t c1rs, c2rs;
+    if (ROWS_ARE_QUERIES) {
+      c1base = reinterpret_cast<const char*>(p.k + batch * p.k_bs + kvh * p.k_hs);
+      c2base = reinterpret_cast<const char*>(p.v + batch * p.v_bs + kvh * p.v_hs);
+      c1rs = (uint32_t)(p.k_rs * 2);
+      c2rs = (uint32_t)(p.v_rs * 2);
+    } else {
+      c1base = reinterpret_cast<const char*>(p.q + batch * p.q_bs + hcol * p.q_hs);
+      c2base = reinterpret_cast<const char*>(p.dout + batch * p.do_bs + hcol * p.do_hs);
+      c1rs = (uint32_t)(p.q_rs * 2);
+      c2rs = (uint32_t)(p.do_rs * 2);
+    }
+    auto col_pos = [&](int c) { return ROWS_ARE_QUERIES ? map.kpos(c) : map.qpos(c); };
+    auto load_tile = [&](int tile, int slot_off) {
+#pragma unroll
+      for (int gi = 0; gi < 2; ++gi) {
+        const int grp = wave * 2 + gi;
+        const int c = im_min(cb + tile * BN + 4 * grp + ld_row, n_cols - 1);
+        const uint32_t pos = col_pos(c);
+        dma_group(c1base + ((uint64_t)pos * c1rs + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
+        dma_group(c2base + ((uint64_t)pos * c2rs + ld_col), lds_base + slot_off + TILE_BYTES + grp * GROUP_STRIDE);
+      }
+    };
+    // column scalars of a tile (dK / dV): wavefront 0 fetches lse * log2(e) and D of its 64 columns
+    float sc_l = 0.f, sc_d = 0.f;
+    auto fetch_scalars = [&](int tile) {
+      if (!ROWS_ARE_QUERIES && wave == 0) {
+        const int c = im_min(cb + tile * BN + lane, n_cols - 1);
+        const int64_t pos = col_pos(c);
+        sc_l = p.lse[batch * p.lse_bs + hcol * p.lse_hs + pos * p.lse_ts] * 1.4426950408889634f;
+        if (MODE == BWD_DK) sc_d = p.dsum[batch * p.ds_bs + hcol * p.ds_hs + pos];
+      }
+    };
+    auto put_scalars = [&](int slot_off) {
+      if (!ROWS_ARE_QUERIES && wave == 0) {
+        float* sc = reinterpret_cast<float*>(smem + slot_off + 2 * TILE_BYTES);
+        sc[lane] = sc_l;
+        sc[64 + lane] = sc_d;
+      }
+    };
+
+    __syncthreads();  // the previous stream's last tile is no longer read
+    if (ntiles > 0) {
+      load_tile(0, 0);
+      fetch_scalars(0);
+      put_scalars(0);
+    }
+    for (int i = 0; i < ntiles; ++i) {
+      const int slot = (i & 1) * BWD_SLOT;
+      tile_barrier<0>();  // tile i has landed for everybody; nobody reads tile i-1 any more
+      if (i + 1 < ntiles) {
+        load_tile(i + 1, BWD_SLOT - slot);
+        fetch_scalars(i + 1);
+      }
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        const int sb_lo = cb + i * BN + 32 * blk;  // first column of the block
+        if (!wave_active || !block_wanted(wb, kpre, sb_lo)) continue;
+        const bool masked = !block_unmasked(wb, kpre, sb_lo);
+        const int c1off = slot + blk * BLOCK32, c2off = slot + TILE_BYTES + blk * BLOCK32;
+        floatx16 s, dp;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) s[e] = dp[e] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kread(c1off, ks), r1f[ks], s, 0, 0, 0);
+        if (MODE != BWD_DV) {
+#pragma unroll
+          for (int ks = 0; ks < 8; ++ks)
+            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kread(c2off, ks), r2f[ks], dp, 0, 0, 0);
+        }
+        // weights: P = exp2(s * c2 - lse2) for visible pairs, dS = P * (dP - D)
+        const float* sc = reinterpret_cast<const float*>(smem + slot + 2 * TILE_BYTES) + 32 * blk + 4 * h32;
+        bf16x8 wp[2];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          floatx4 l4 = {L2_row, L2_row, L2_row, L2_row}, d4 = {D_row, D_row, D_row, D_row};
+          if (!ROWS_ARE_QUERIES) {
+            l4 = *reinterpret_cast<const floatx4*>(sc + 8 * t);
+            if (MODE == BWD_DK) d4 = *reinterpret_cast<const floatx4*>(sc + 64 + 8 * t);
+          }
+          float w[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int e = 4 * t + u;
+            const int col = sb_lo + 8 * t + 4 * h32 + u;
+            float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c2, -l4[u]));
+            if (masked && !key_visible(col, kpre, lo_l, hi_l)) x = 0.f;
+            if (MODE != BWD_DV) x *= dp[e] - d4[u];
+            w[u] = x;
+          }
+          floatx2 f0 = {w[0], w[1]}, f1 = {w[2], w[3]};
+          bf16x2 h0 = __builtin_convertvector(f0, bf16x2), h1 = __builtin_convertvector(f1, bf16x2);
+          wp[t >> 1][4 * (t & 1) + 0] = h0[0];
+          wp[t >> 1][4 * (t & 1) + 1] = h0[1];
+          wp[t >> 1][4 * (t & 1) + 2] = h1[0];
+          wp[t >> 1][4 * (t & 1) + 3] = h1[1];
+        }
+        const int xoff = MODE == BWD_DV ? c2off : c1off;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vread(xoff, j), wp[j >> 2], acc[j & 3], 0, 0, 0);
+      }
+      if (i + 1 < ntiles) put_scalars(BWD_SLOT - slot);
+    }
+  }
+
+  // ---------------------------------------------------------------- scale, round, store
+  if (!wave_active) return;
+  const float f = MODE == BWD_DV ? 1.f : p.scale;
+  uint16_t* orow;
+  if (MODE == BWD_DQ) orow = p.dq + (batch * p.dq_bs + rpos * p.dq_rs + hq * p.dq_hs + 8 * h32);
+  else if (MODE == BWD_DK) orow = p.dk + (batch * p.dk_bs + rpos * p.dk_rs + kvh * p.dk_hs + 8 * h32);
+  else orow = p.dv + (batch * p.dv_bs + rpos * p.dv_rs + kvh * p.dv_hs + 8 * h32);
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int g2 = 0; g2 < 2; ++g2) {
+      uint32_t w[4];
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          const int e = 8 * g2 + 4 * half + 2 * k;
+          floatx2 v2 = {acc[db][e] * f, acc[db][e + 1] * f};
+          w[2 * half + k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
+        }
+      auto q0 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+      auto q1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+      if (row_valid) {
+        u32x4 pk = {q0[0], q1[0], q0[1], q1[1]};
+        *reinterpret_cast<u32x4*>(orow + 32 * db + 16 * g2) = pk;
+      }
+    }
+}
+
+}  // namespace intra

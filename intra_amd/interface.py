@@ -126,6 +126,61 @@ def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_
                    int(window), _scale(q, softmax_scale), return_lse)
 
 
+def intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", group_num=8, window=576, softmax_scale=None,
+                       block=256):
+    """Gradients (dq, dk, dv) of intra_llm_attn for pattern "scatter", "gather1", "window" or
+    "block_scatter" (offset 0, no sinks), given the forward results `out`, `lse` (return_lse=True)
+    and the gradient `dout` of `out`.  The reference has no backward kernels (its training runs
+    differentiate masked SDPA, experiments/llm/llama_intra.py:26)."""
+    q, k, v = _check(q, k, v)
+    ids = dict(LLM_PATTERNS, block_scatter=EXTRA_LLM_PATTERNS["block_scatter"])
+    if pattern not in ids:
+        raise ValueError(f"no backward kernels for pattern {pattern!r}")
+    if pattern == "gather1" and (group_num != 8 or q.shape[1] % (group_num * group_num)):
+        raise ValueError(f"gather1 needs group_num=8 and seqlen % 64 == 0, got G={group_num}, S={q.shape[1]}")
+    fix = lambda t: t if (t.stride(-1) == 1 and _aligned(t)) else t.contiguous()
+    out, dout = fix(out), fix(dout)
+    if out.shape != q.shape or dout.shape != q.shape or out.dtype != q.dtype or dout.dtype != q.dtype:
+        raise ValueError("out and dout must have the shape and dtype of q")
+    B, S, H, _ = q.shape
+    if lse.shape != (B, H, S) or lse.dtype != torch.float32:
+        raise ValueError("lse must be the (batch, heads, seqlen) fp32 tensor of the forward call")
+    dq, dk, dv = (torch.empty(t.shape, dtype=t.dtype, device=t.device) for t in (q, k, v))
+    work = torch.empty(B, H, S, dtype=torch.float32, device=q.device)
+    guard, stream = _stream_on(q.device)
+    with guard:
+        rc = _C.intra_llm_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), dout.data_ptr(),
+                              dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), work.data_ptr(), B, S, H, k.shape[2],
+                              _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                              _lib.strides3(dout), _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv),
+                              _lib.strides3(lse), ids[pattern], int(group_num), int(window), int(block), 0, 0,
+                              float(_scale(q, softmax_scale)), stream)
+    if rc != _lib.INTRA_OK:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
+    return dq, dk, dv
+
+
+class _LlmAttnFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, pattern, group_num, window, softmax_scale, block):
+        out, lse = intra_llm_attn(q, k, v, pattern, group_num, window, softmax_scale, return_lse=True, block=block)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.args = (pattern, group_num, window, softmax_scale, block)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        dq, dk, dv = intra_llm_attn_bwd(q, k, v, out, lse, dout, *ctx.args)
+        return dq, dk, dv, None, None, None, None, None
+
+
+def intra_llm_attn_func(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None, block=256):
+    """intra_llm_attn as a differentiable function (torch.autograd) for the patterns that
+    intra_llm_attn_bwd covers."""
+    return _LlmAttnFunction.apply(q, k, v, pattern, group_num, window, softmax_scale, block)
+
+
 def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None, return_lse=False):
     """Bidirectional attention for FLUX-style sequences: 512 text tokens followed by a
     width x width grid of image tokens.

@@ -32,12 +32,16 @@ What it restates (reference file:line) and what pins each function (tests/test_o
   attention.masked_attention intra_attn/reference.py:78-83   float64 triple loop on tiny inputs;
                                                               torch SDPA (the library routine the
                                                               reference calls) incl. GQA
+  attention.masked_attention_grads   experiments/llm/llama_intra.py:26 (autograd of masked SDPA)
+                                                              central finite differences in float64;
+                                                              hand-written softmax-Jacobian formulas in
+                                                              loops; closed form for one-key rows
   pairs.*                    closed forms                     mask.sum() of the masks above
 
 Every function has at least one such independent check, so no part is "parity unpinned".
 The reference's Python file was read, not imported or run.
 """
-from .attention import masked_attention, masked_attention_rows, masked_lse_rows  # noqa: F401
+from .attention import masked_attention, masked_attention_grads, masked_attention_rows, masked_lse_rows  # noqa: F401
 from .masks import (TEXT_LEN, image_gather0_mask, image_scatter_mask, llm_block_scatter_mask,  # noqa: F401
                     llm_gather1_mask, llm_scatter_mask, llm_window_mask, llm_window_sink_mask, mask_rows)
 from .pairs import pairs_per_head  # noqa: F401

@@ -63,3 +63,23 @@ def masked_lse_rows(q, k, mask_rows, rows=None, softmax_scale=None, chunk=1024):
 def masked_attention(q, k, v, mask, softmax_scale=None, chunk=1024):
     """reference.py:78-83: q, k, v (B, S, H, D) with H % Hkv == 0; mask (S, S) bool."""
     return masked_attention_rows(q, k, v, mask, None, softmax_scale, chunk)
+
+
+def masked_attention_grads(q, k, v, dout, mask, softmax_scale=None, dtype=torch.float32):
+    """Gradients (dq, dk, dv) of sum(masked_attention(q, k, v, mask) * dout) with respect to q, k
+    and v, by automatic differentiation of the explicit matmul / softmax formulation in `dtype`.
+    The reference differentiates the same dense-mask attention in its training experiments
+    (experiments/llm/llama_intra.py:26: masked SDPA under autograd); it has no backward kernels.
+    q, dout: (B, S, H, D); k, v: (B, S, Hkv, D); mask: (S, S) bool.  Results in `dtype`."""
+    B, S, H, D = q.shape
+    Hkv = k.shape[2]
+    rep = H // Hkv
+    scale = D ** -0.5 if softmax_scale is None else softmax_scale
+    with torch.enable_grad():
+        qf, kf, vf = (t.detach().to(dtype).requires_grad_(True) for t in (q, k, v))
+        qh = qf.permute(0, 2, 1, 3).reshape(B, Hkv, rep, S, D)
+        s = torch.matmul(qh, kf.permute(0, 2, 3, 1)[:, :, None]) * scale
+        s = s.masked_fill(~mask.to(q.device)[None, None, None], float("-inf"))
+        o = torch.matmul(torch.softmax(s, dim=-1), vf.permute(0, 2, 1, 3)[:, :, None])
+        o = o.reshape(B, H, S, D).permute(0, 2, 1, 3)
+        return torch.autograd.grad(o, (qf, kf, vf), dout.detach().to(dtype))

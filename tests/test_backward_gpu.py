@@ -1,0 +1,143 @@
+"""Parity of the backward kernels (dq, dk, dv through intra_llm_bwd of the C ABI) against the
+gradients of the fp32 dense-mask oracle.  The reference has no backward kernels; what it
+differentiates in training is the dense-mask attention the oracle restates
+(experiments/llm/llama_intra.py:26), so that is the specification.
+
+Tolerance, on bf16 results, per tensor with m = max|want|:
+  every element  |got - want| <= m / 64 + |want| / 64
+  whole tensor   ||got - want||_2 <= ||want||_2 / 128
+The kernels round the softmax weights and their derivatives to bf16 before the second product
+(2^-9 relative each), use the forward pass's log-sum-exp (within 2^-8 of exact), form
+D = dout . out from the bf16 output, and round the results to bf16 (2^-9).  The terms that add up
+to one gradient element partly cancel, so an element's error scales with the tensor, not with the
+element: hence the m / 64.  The norm bound is the sharp one: a dropped term, a wrong scale or a
+missed key block moves it by orders of magnitude."""
+import pytest
+import torch
+
+import oracle
+from intra_amd import intra_llm_attn, intra_llm_attn_bwd, intra_llm_attn_func
+
+pytestmark = pytest.mark.gpu
+RTOL, NORM_RTOL = 1.0 / 64, 1.0 / 128
+DEV = "cuda"
+
+
+def make(B, S, H, Hkv, seed=0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    mk = lambda h: torch.randn(B, S, h, 128, generator=g, dtype=torch.float32).to(torch.bfloat16).to(DEV)
+    return mk(H), mk(Hkv), mk(Hkv), mk(H)
+
+
+def kernel_grads(q, k, v, dout, pattern, scale=None, **kw):
+    with torch.no_grad():
+        out, lse = intra_llm_attn(q, k, v, pattern, softmax_scale=scale, return_lse=True, **kw)
+        return intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern, softmax_scale=scale, **kw)
+
+
+def compare(got, want, what):
+    for name, g, w in zip(("dq", "dk", "dv"), got, want):
+        assert g.dtype == torch.bfloat16 and g.shape == w.shape
+        assert bool(torch.isfinite(g).all()), f"{what} {name} not finite"
+        w = w.float()
+        diff = (g.float() - w).abs()
+        m = w.abs().max().item()
+        ok = diff <= RTOL * m + RTOL * w.abs()
+        assert bool(ok.all()), f"{what} {name}: max|err|={diff.max().item():.3e}, max|want|={m:.3e}"
+        rel = (diff.norm() / w.norm()).item()
+        assert rel <= NORM_RTOL, f"{what} {name}: relative l2 error {rel:.3e}"
+
+
+def run_case(kind, pattern, B, S, H, Hkv, seed=0, scale=None, mask_kw=None, **kw):
+    q, k, v, dout = make(B, S, H, Hkv, seed)
+    got = kernel_grads(q, k, v, dout, pattern, scale, **kw)
+    mask = oracle.mask_rows(kind, S, device=DEV, **(mask_kw if mask_kw is not None else kw))
+    want = oracle.masked_attention_grads(q, k, v, dout, mask, softmax_scale=scale)
+    compare(got, want, f"{kind} S={S} H={H}/{Hkv} {kw}")
+
+
+@pytest.mark.parametrize("S", [63, 777, 1024, 4096])
+@pytest.mark.parametrize("G", [2, 3, 8])
+@pytest.mark.parametrize("B,H,Hkv", [(1, 8, 2), (2, 4, 4), (1, 6, 3)])
+def test_scatter_grads(S, G, B, H, Hkv):
+    run_case("llm/scatter", "scatter", B, S, H, Hkv, group_num=G)
+
+
+@pytest.mark.parametrize("S", [64, 1024, 2112])
+@pytest.mark.parametrize("B,H,Hkv", [(1, 8, 2), (2, 4, 4)])
+def test_gather1_grads(S, B, H, Hkv):
+    run_case("llm/gather1", "gather1", B, S, H, Hkv, group_num=8)
+
+
+@pytest.mark.parametrize("S,W", [(300, 64), (2000, 576), (3000, 1000), (1000, 4096)])
+@pytest.mark.parametrize("B,H,Hkv", [(1, 8, 2), (2, 2, 2)])
+def test_window_grads(S, W, B, H, Hkv):
+    run_case("llm/window", "window", B, S, H, Hkv, window=W)
+
+
+@pytest.mark.parametrize("S,G,block", [(1500, 2, 256), (1111, 3, 64), (4096, 2, 256), (700, 4, 128)])
+@pytest.mark.parametrize("B,H,Hkv", [(1, 8, 2), (1, 4, 1)])
+def test_block_scatter_grads(S, G, block, B, H, Hkv):
+    run_case("llm/block_scatter", "block_scatter", B, S, H, Hkv, group_num=G, block=block)
+
+
+def test_headline_heads_at_8k():
+    run_case("llm/scatter", "scatter", 1, 8192, 32, 8, group_num=8)
+
+
+def test_other_scale():
+    run_case("llm/scatter", "scatter", 1, 1000, 8, 2, scale=0.05, group_num=4)
+
+
+def test_strided_inputs_and_packed_qkv():
+    # q, k, v as slices of one packed projection output; dout a transposed view
+    B, S, H, Hkv = 1, 1024, 8, 2
+    g = torch.Generator(device="cpu").manual_seed(4)
+    qkv = torch.randn(B, S, H + 2 * Hkv, 128, generator=g).to(torch.bfloat16).to(DEV)
+    q, k, v = qkv[:, :, :H], qkv[:, :, H:H + Hkv], qkv[:, :, H + Hkv:]
+    dout = torch.randn(B, H, S, 128, generator=g).to(torch.bfloat16).to(DEV).transpose(1, 2)
+    got = kernel_grads(q, k, v, dout, "scatter", group_num=8)
+    want = oracle.masked_attention_grads(q, k, v, dout, oracle.llm_scatter_mask(S, 8, DEV))
+    compare(got, want, "packed qkv")
+
+
+def test_full_length_properties():
+    """At S = 32768 (headline shape) the dense oracle is out of reach; properties that hold for
+    any size: the gradients are linear in dout; dv of an all-ones dout sums the weights (every
+    query's weights add to one, so the sum over keys of dv is the number of queries per kv head);
+    the first token of each group sees only itself, so its weight is 1 and its dq vanishes (up to
+    the fp32 rounding of dP - D, both of which equal dout . v there)."""
+    B, S, H, Hkv, G = 1, 32768, 32, 8, 8
+    q, k, v, dout = make(B, S, H, Hkv, seed=9)
+    with torch.no_grad():
+        out, lse = intra_llm_attn(q, k, v, "scatter", group_num=G, return_lse=True)
+        d1 = intra_llm_attn_bwd(q, k, v, out, lse, dout, "scatter", group_num=G)
+        d2 = intra_llm_attn_bwd(q, k, v, out, lse, dout * 2, "scatter", group_num=G)  # exact in bf16
+        for a, b in zip(d1, d2):
+            assert torch.equal(a.float() * 2, b.float())
+        ones = torch.ones_like(dout)
+        dq1, dk1, dv1 = intra_llm_attn_bwd(q, k, v, out, lse, ones, "scatter", group_num=G)
+        total = dv1.float().sum(dim=1)  # (B, Hkv, 128): sum over keys
+        assert (total / (S * H // Hkv) - 1).abs().max().item() < 4e-3
+        assert d1[0][:, :G].float().abs().max().item() < 1e-3
+        assert bool(torch.isfinite(dk1).all()) and bool(torch.isfinite(dq1).all())
+
+
+def test_autograd_function_matches_dense_autograd():
+    B, S, H, Hkv = 1, 1024, 8, 2
+    q, k, v, _ = make(B, S, H, Hkv, seed=2)
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    out = intra_llm_attn_func(q, k, v, "scatter", 8)
+    w = torch.linspace(-1, 1, 128, device=DEV)
+    (out.float() * w).sum().backward()
+    dout = w.expand_as(out).to(torch.bfloat16)
+    want = oracle.masked_attention_grads(q, k, v, dout, oracle.llm_scatter_mask(S, 8, DEV))
+    compare((q.grad, k.grad, v.grad), want, "autograd")
+
+
+def test_unsupported_patterns_raise():
+    q, k, v, dout = make(1, 512, 4, 4)
+    with torch.no_grad():
+        out, lse = intra_llm_attn(q, k, v, "window_sink", window=100, n_sink=4, return_lse=True)
+    with pytest.raises(ValueError):
+        intra_llm_attn_bwd(q, k, v, out, lse, dout, "window_sink", window=100)

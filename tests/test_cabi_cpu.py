@@ -220,3 +220,30 @@ def test_ex_argument_checks(lib):
     assert lib.intra_plan_llm_ex(0, 1, 32768, 32, 8, 8, 576, 0, 0, 0, ctypes.byref(p)) == 0
     assert lib.intra_plan(0, 0, 1, 32768, 32, 8, 8, 576, ctypes.byref(q)) == 0
     assert (p.work_items, p.pairs_per_head) == (q.work_items, q.pairs_per_head)
+
+
+def test_bwd_validates_before_touching_the_gpu(lib):
+    st = _lib._i64x3(512 * 4 * 128, 4 * 128, 128)
+    ls = _lib._i64x3(4 * 512, 512, 1)
+    P = 0x1000  # never dereferenced: every call below fails validation first
+
+    def call(ptrs=(P,) * 10, B=1, S=512, H=4, Hkv=4, strides=(st,) * 8, lse_strides=ls, pattern=0, G=2, window=576,
+             block=256, offset=0, n_sink=0, scale=0.1):
+        return lib.intra_llm_bwd(*ptrs, B, S, H, Hkv, *strides, lse_strides, pattern, G, window, block, offset, n_sink,
+                                 scale, None)
+
+    for i in range(10):  # q, k, v, o, lse, dout, dq, dk, dv, workspace
+        assert call(ptrs=tuple(None if j == i else P for j in range(10))) == _lib.INTRA_ERR_INVALID
+        assert "non-null" in _lib.last_error()
+    assert call(ptrs=(P + 8,) + (P,) * 9) == _lib.INTRA_ERR_INVALID and "16-byte aligned" in _lib.last_error()
+    assert call(ptrs=(P,) * 4 + (P + 2,) + (P,) * 5) == _lib.INTRA_ERR_INVALID and "4-byte aligned" in _lib.last_error()
+    odd = _lib._i64x3(512 * 4 * 128, 4 * 128 + 4, 128)
+    assert call(strides=(st,) * 4 + (odd,) + (st,) * 3) == _lib.INTRA_ERR_INVALID and "dout" in _lib.last_error()
+    assert call(scale=float("nan")) == _lib.INTRA_ERR_INVALID
+    assert call(H=6, Hkv=4) == _lib.INTRA_ERR_INVALID
+    assert call(pattern=7) == _lib.INTRA_ERR_INVALID
+    # patterns whose dk / dv are not built
+    assert call(pattern=9, window=100) == _lib.INTRA_ERR_UNSUPPORTED
+    assert call(pattern=8, offset=1) == _lib.INTRA_ERR_UNSUPPORTED
+    assert call(pattern=8, n_sink=4) == _lib.INTRA_ERR_UNSUPPORTED
+    assert "backward" in _lib.last_error()

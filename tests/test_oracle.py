@@ -387,3 +387,65 @@ def test_reference_known_answers():
                 assert bool(m[q, k]) == bool(eval(entry["rule"], {"q": q, "k": k, "G": G}))
     for entry in data["pairs"]:
         assert pairs.pairs_per_head(entry["kind"], entry["S"], **entry["args"]) == entry["pairs_per_head"]
+
+
+# ---------------------------------------------------------------------------- gradients
+def _tiny_problem(seed, S=12, H=4, Hkv=2, D=8):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda h: torch.randn(1, S, h, D, generator=g, dtype=torch.float64)
+    return mk(H), mk(Hkv), mk(Hkv), mk(H)
+
+
+def test_grads_match_finite_differences():
+    # central differences of the scalar sum(O * dout) in float64, every input element
+    q, k, v, dout = _tiny_problem(3, S=6, H=2, Hkv=1, D=4)
+    mask = masks.llm_scatter_mask(6, 2)
+    grads = oracle.masked_attention_grads(q, k, v, dout, mask, dtype=torch.float64)
+    sdpa = lambda a, b, c: F.scaled_dot_product_attention(a.transpose(1, 2), b.transpose(1, 2), c.transpose(1, 2),
+                                                          attn_mask=mask, enable_gqa=True).transpose(1, 2)
+    f = lambda a, b, c: (sdpa(a, b, c) * dout).sum().item()  # the library routine, in float64
+    eps = 1e-5
+    for which, (x, gx) in enumerate(zip((q, k, v), grads)):
+        flat = x.reshape(-1)
+        for i in range(flat.numel()):
+            old = flat[i].item()
+            flat[i] = old + eps
+            up = f(q, k, v)
+            flat[i] = old - eps
+            dn = f(q, k, v)
+            flat[i] = old
+            assert abs((up - dn) / (2 * eps) - gx.reshape(-1)[i].item()) < 1e-6, (which, i)
+
+
+def test_grads_match_the_softmax_jacobian_formulas():
+    # dV = P^T dO, dS = P o (dP - rowsum(dO o O)), dQ = scale dS K, dK = scale dS^T Q, in plain loops
+    q, k, v, dout = _tiny_problem(5)
+    S, H, Hkv, D = 12, 4, 2, 8
+    mask = masks.llm_window_mask(S, 4) | torch.eye(S, dtype=torch.bool)
+    scale = 0.3
+    dq, dk, dv = oracle.masked_attention_grads(q, k, v, dout, mask, softmax_scale=scale, dtype=torch.float64)
+    eq, ek, ev = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    for h in range(H):
+        kv = h // (H // Hkv)
+        for i in range(S):
+            js = [j for j in range(S) if mask[i, j]]
+            s = torch.tensor([scale * float(q[0, i, h] @ k[0, j, kv]) for j in js], dtype=torch.float64)
+            p = torch.exp(s - torch.logsumexp(s, 0))
+            o = sum(p[n] * v[0, j, kv] for n, j in enumerate(js))
+            dsum = float(dout[0, i, h] @ o)
+            for n, j in enumerate(js):
+                ev[0, j, kv] += p[n] * dout[0, i, h]
+                ds = p[n] * (float(dout[0, i, h] @ v[0, j, kv]) - dsum)
+                eq[0, i, h] += scale * ds * k[0, j, kv]
+                ek[0, j, kv] += scale * ds * q[0, i, h]
+    for got, want in ((dq, eq), (dk, ek), (dv, ev)):
+        assert (got - want).abs().max().item() < 1e-10
+
+
+def test_grads_of_one_key_rows_have_a_closed_form():
+    # a query that sees a single key has P = 1: dV gets dO, dQ and dK get nothing
+    q, k, v, dout = _tiny_problem(7, H=2, Hkv=2)
+    mask = torch.eye(12, dtype=torch.bool)
+    dq, dk, dv = oracle.masked_attention_grads(q, k, v, dout, mask, dtype=torch.float64)
+    assert dq.abs().max().item() < 1e-12 and dk.abs().max().item() < 1e-12
+    assert (dv - dout).abs().max().item() < 1e-12
