@@ -15,7 +15,7 @@ import json
 import torch
 import torch.nn.functional as F
 
-from intra_amd import _lib, intra_image_attn, intra_llm_attn
+from intra_amd import _lib, intra_image_attn, intra_llm_attn, intra_llm_attn_bwd
 from intra_amd.interface import TEXT_LEN
 
 PEAK_BF16_TFLOPS = 2516.6
@@ -106,6 +106,21 @@ def bench_llm(args):
                     else:
                         intra_llm_attn(ql, kl, vl, "window", window=576)
             r["g2s4_32layer_run"] = round(median_ms(stack, 2, max(3, args.iters // 10)), 3)
+        if args.backward:
+            # dq, dk, dv of the same calls (three launches); flops counted as 5 products per pair
+            # (S, dP, dV, dQ, dK), i.e. 2.5 x the forward's, whatever the kernels recompute
+            dout = qkv(B, S, H, Hkv, seed=1)[0]
+            cases = [(f"scatter_g{G}", "scatter", dict(group_num=G), pairs(0, 0, B, S, H, Hkv, G, 576)) for G in args.groups]
+            if S % 64 == 0:
+                cases.append(("gather1_g8", "gather1", dict(group_num=8), pairs(0, 1, B, S, H, Hkv, 8, 576)))
+            cases.append(("window576", "window", dict(window=576), pairs(0, 4, B, S, H, Hkv, 8, 576)))
+            for key, pattern, kw, npairs in cases:
+                out, lse = intra_llm_attn(q, k, v, pattern, return_lse=True, **kw)
+                ms = median_ms(lambda: intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern, **kw), args.warmup, args.iters)
+                tf = 10 * 128 * npairs * H * B / (ms * 1e-3) / 1e12
+                r[key + "_bwd"] = round(ms, 4)
+                r[key + "_bwd_tflops"] = round(tf, 1)
+                r[key + "_bwd_pct_peak"] = round(100 * tf / PEAK_BF16_TFLOPS, 1)
         if args.model_patterns:
             # the layers the reference's model integration really runs in its g2s4 LLaMA setting
             # (experiments/llm/llama_intra.py:16-18): block Scatter with 2 groups of 256-token
@@ -164,6 +179,7 @@ def main():
     p.add_argument("--dense", action="store_true", help="also time torch SDPA on the dense problem")
     p.add_argument("--model-patterns", action="store_true",
                    help="llm: also time block Scatter and window-with-sinks layers (g2s4 model setting)")
+    p.add_argument("--backward", action="store_true", help="llm: also time the backward pass (dq, dk, dv) of each pattern")
     p.add_argument("--out", help="optional JSON output path")
     args = p.parse_args()
     args.seqlens = [int(x) for x in args.seqlens.split(",")]

@@ -395,6 +395,16 @@ int launch_bwd(const intra::BParams& p, int64_t grid, hipStream_t stream) {
   return INTRA_OK;
 }
 
+// Grid of one backward launch: per XCD, bundles of pairs x items of a pair (see the kernel).
+int64_t bwd_grid(intra::BParams& p, int64_t pairs) {
+  p.items_per_pair = p.n_rblocks * p.hgroups;
+  const int64_t pairs_per_xcd = (pairs + 7) / 8;
+  const int64_t want = (32 + p.items_per_pair - 1) / p.items_per_pair;  // pairs that fill an XCD's 32 CUs
+  p.bundle = (int)std::max<int64_t>(1, std::min<int64_t>(want, pairs_per_xcd));
+  const int64_t bundles = (pairs_per_xcd + p.bundle - 1) / p.bundle;
+  return 8 * bundles * p.bundle * p.items_per_pair;
+}
+
 template <class MAP>
 int run_bwd_map(intra::BParams p, int hp, const Request& r, hipStream_t stream) {
   const int64_t pairs = (int64_t)MAP::num_sets(p.geom) * r.B * r.Hkv;
@@ -402,18 +412,20 @@ int run_bwd_map(intra::BParams p, int hp, const Request& r, hipStream_t stream) 
   // dQ: row blocks of 256 / hp queries of hp heads; writes D = rowsum(dO o O) for the dK launch
   p.hgroups = (r.H / r.Hkv) / hp;
   p.n_rblocks = (max_rows + 256 / hp - 1) / (256 / hp);
+  int64_t grid = bwd_grid(p, pairs);
   int rc;
   switch (hp) {
-    case 4: rc = launch_bwd<MAP, intra::BWD_DQ, 4>(p, pairs * p.n_rblocks * p.hgroups, stream); break;
-    case 2: rc = launch_bwd<MAP, intra::BWD_DQ, 2>(p, pairs * p.n_rblocks * p.hgroups, stream); break;
-    default: rc = launch_bwd<MAP, intra::BWD_DQ, 1>(p, pairs * p.n_rblocks * p.hgroups, stream); break;
+    case 4: rc = launch_bwd<MAP, intra::BWD_DQ, 4>(p, grid, stream); break;
+    case 2: rc = launch_bwd<MAP, intra::BWD_DQ, 2>(p, grid, stream); break;
+    default: rc = launch_bwd<MAP, intra::BWD_DQ, 1>(p, grid, stream); break;
   }
   if (rc) return rc;
   // dK, dV: row blocks of 256 keys of one kv head, all query heads of its group streamed past
   p.hgroups = 1;
   p.n_rblocks = (max_rows + 255) / 256;
-  if ((rc = launch_bwd<MAP, intra::BWD_DK, 1>(p, pairs * p.n_rblocks, stream))) return rc;
-  return launch_bwd<MAP, intra::BWD_DV, 1>(p, pairs * p.n_rblocks, stream);
+  grid = bwd_grid(p, pairs);
+  if ((rc = launch_bwd<MAP, intra::BWD_DK, 1>(p, grid, stream))) return rc;
+  return launch_bwd<MAP, intra::BWD_DV, 1>(p, grid, stream);
 }
 
 int run_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
@@ -442,6 +454,7 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
     return rc;
   if (!ls) return fail(INTRA_ERR_INVALID, "lse strides pointer is null");
   if (!isfinite(scale)) return fail(INTRA_ERR_INVALID, "softmax_scale must be finite");
+  if (scale == 0.f) return fail(INTRA_ERR_UNSUPPORTED, "backward: softmax_scale must not be zero");
   const int64_t* all[] = {qs, ks, vs, dos};
   for (const int64_t* st : all)
     if (st[1] >= ((int64_t)1 << 31)) return fail(INTRA_ERR_UNSUPPORTED, "token strides must stay below 2^31 elements");

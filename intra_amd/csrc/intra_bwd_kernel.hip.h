@@ -1,6 +1,6 @@
-// Backward kernels of the sparse attention for gfx950 (MI355X): dQ for every pattern, dK / dV for
-// the patterns whose sets number queries and keys alike (LLM Scatter, Gather 1, 64-aligned window,
-// block Scatter without offset and sinks).
+// Backward kernels of the sparse attention for gfx950 (MI355X): dQ, dK and dV for the patterns
+// whose sets number queries and keys alike and whose rows meet one contiguous range of columns
+// (LLM Scatter, Gather 1, 64-aligned window, block Scatter without offset and sinks).
 //
 // The reference has no backward kernels (its README names them as missing; training there runs
 // through masked SDPA / FlexAttention, experiments/llm/llama_intra.py:26).  The math is the usual
@@ -10,7 +10,7 @@
 // One template serves the three results.  A workgroup owns 256 / HP "rows" (queries for dQ, keys
 // for dK and dV; 32 per wavefront, held as MFMA B operands in registers like Q in the forward
 // kernel) and streams the "columns" that see them through LDS in tiles of 64 (K and V rows for
-// dQ, Q and dO rows of every query head of the group for dK / dV), double buffered.  Per 32
+// dQ, Q and dO rows of every query head of the group for dK / dV) through three slots.  Per 32
 // columns a wavefront forms the scores S^T = C1 R1^T and dP^T = C2 R2^T, turns them into the
 // weights (P or dS), packed to bf16 straight from the accumulators, and adds X^T W^T to its
 // accumulators, X being the K, Q or dO tile read with transposing LDS reads - the data flow of
@@ -41,17 +41,19 @@ struct BParams {
   float scale_log2;  // scale * log2(e)
   int n_rblocks;     // row blocks per set
   int hgroups;       // ratio / HP (dQ only)
+  int items_per_pair;  // n_rblocks * hgroups
+  int bundle;        // pairs of one XCD that are worked on together
 };
 
 constexpr int BWD_SLOT = 2 * TILE_BYTES + 512;  // two tiles and 2 x 64 column scalars
-constexpr int BWD_LDS_BYTES = 2 * BWD_SLOT;
+constexpr int BWD_LDS_BYTES = 3 * BWD_SLOT;
 
 template <class MAP, int MODE, int HP>
 __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   constexpr int NW = 8;
   constexpr bool ROWS_ARE_QUERIES = MODE == BWD_DQ;
   constexpr int POS = ROWS_ARE_QUERIES ? NW * 32 / HP : NW * 32;  // rows per row block (of one head)
-  static_assert(ROWS_ARE_QUERIES || !MAP::kHasPrefix, "dK / dV need a per-set key numbering without prefix");
+  static_assert(!MAP::kHasPrefix, "built for maps whose rows meet one contiguous range of columns");
 
   __shared__ __attribute__((aligned(1024))) unsigned char smem[BWD_LDS_BYTES];
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
@@ -63,15 +65,23 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   const int l32 = lane & 31;
 
   // ---------------------------------------------------------------- work item
-  int item = blockIdx.x;
-  int hg = 0;
-  if (ROWS_ARE_QUERIES) {
-    hg = item % p.hgroups;
-    item /= p.hgroups;
-  }
-  const int rblk = item % p.n_rblocks;
-  const int pair = item / p.n_rblocks;
+  // Workgroups start in blockIdx order, round-robin over the 8 XCDs, and a CU takes the next one
+  // when it has finished one.  Per XCD the (set, batch, kv head) pairs are taken in bundles of
+  // `bundle` pairs - as few as fill its 32 CUs - so that the workgroups running together stream the
+  // same few megabytes of columns through the XCD's L2; within a bundle the row blocks with the
+  // most columns come first (the last query blocks for dQ, the first key blocks for dK / dV).
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int per_bundle = p.bundle * p.items_per_pair;
+  const int bun = slot / per_bundle, rem = slot - bun * per_bundle;
+  const int heavy = rem / p.bundle;
   const int nbh = p.B * p.Hkv;
+  const int pair = (bun * p.bundle + (rem - heavy * p.bundle)) * 8 + xcd;
+  if (pair >= MAP::num_sets(p.geom) * nbh) return;
+  int hg = 0, rblk = heavy;
+  if (ROWS_ARE_QUERIES) {
+    hg = heavy % p.hgroups;
+    rblk = p.n_rblocks - 1 - heavy / p.hgroups;
+  }
   const int set = pair / nbh;
   const int bh = pair % nbh;
   const int batch = bh / p.Hkv;
@@ -109,7 +119,7 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
     return lo;
   };
 
-  const int cb = (ROWS_ARE_QUERIES && MAP::kHasPrefix) ? 0 : col_lo(r0);  // first column of the row block
+  const int cb = col_lo(r0);  // first column of the row block
   const int ce = col_hi(r1);                                             // last one
   const int ntiles = ce >= cb ? (ce - cb + BN) / BN : 0;
 
@@ -126,6 +136,9 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   wb.w_hi = __builtin_amdgcn_readfirstlane(col_hi(wr_last));
   wb.f_lo = __builtin_amdgcn_readfirstlane(col_lo(wr_last));
   wb.f_hi = __builtin_amdgcn_readfirstlane(col_hi(im_min(wr0, r1)));
+  // the blocks of 32 columns (counted from cb) that this wavefront's rows meet: one range
+  const int jb_lo = wave_active ? (wb.w_lo - cb) >> 5 : 1;
+  const int jb_hi = wave_active ? (wb.w_hi - cb) >> 5 : 0;
   const int64_t rpos = ROWS_ARE_QUERIES ? map.qpos(row) : map.kpos(row);
   const int hq = kvh * p.ratio + hg * HP + hw;  // query head of a query row
 
@@ -192,117 +205,203 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
   const float c2 = p.scale_log2;
+  const float s_hidden = c2 >= 0.f ? -INFINITY : INFINITY;  // score that gives exp2(s * c2 - lse) = 0
 
-  // ---------------------------------------------------------------- column streams
-  // dQ: one stream (the K / V rows of the kv head); dK, dV: one per query head of the group.
+  // ---------------------------------------------------------------- column steps
+  // dQ meets one stream of columns (the K / V rows of the kv head), tile after tile from the first.
+  // dK / dV meet one per query head of the group (its Q / dO rows); they take the tiles from the
+  // last one down and, per tile, head after head: all key blocks of a (set, batch, kv head) start
+  // at the last tile together and stay in step, so that a tile fetched for one of them is in the
+  // L2 for the others.  A step is one (tile, head).
   const int n_streams = ROWS_ARE_QUERIES ? 1 : p.ratio;
-  for (int sidx = 0; sidx < n_streams; ++sidx) {
-    const int hcol = kvh * p.ratio + sidx;  // query head of the columns (dK / dV)
-    const char *c1base, *c2base;
-    uint32_t c1rs, c2rs;
+  const int n_steps = ntiles * n_streams;
+  struct Cursor {
+    int tile, head;
+  };
+  auto advance = [&](Cursor& c) {
     if (ROWS_ARE_QUERIES) {
-      c1base = reinterpret_cast<const char*>(p.k + batch * p.k_bs + kvh * p.k_hs);
-      c2base = reinterpret_cast<const char*>(p.v + batch * p.v_bs + kvh * p.v_hs);
-      c1rs = (uint32_t)(p.k_rs * 2);
-      c2rs = (uint32_t)(p.v_rs * 2);
-    } else {
-      c1base = reinterpret_cast<const char*>(p.q + batch * p.q_bs + hcol * p.q_hs);
-      c2base = reinterpret_cast<const char*>(p.dout + batch * p.do_bs + hcol * p.do_hs);
-      c1rs = (uint32_t)(p.q_rs * 2);
-      c2rs = (uint32_t)(p.do_rs * 2);
+      ++c.tile;
+    } else if (++c.head == n_streams) {
+      c.head = 0;
+      --c.tile;
     }
-    auto col_pos = [&](int c) { return ROWS_ARE_QUERIES ? map.kpos(c) : map.qpos(c); };
-    auto load_tile = [&](int tile, int slot_off) {
+  };
+  const char *c1base, *c2base;
+  uint32_t c1rs, c2rs;
+  int64_t c1hs = 0, c2hs = 0;  // byte stride between the heads of the group (dK / dV)
+  if (ROWS_ARE_QUERIES) {
+    c1base = reinterpret_cast<const char*>(p.k + batch * p.k_bs + kvh * p.k_hs);
+    c2base = reinterpret_cast<const char*>(p.v + batch * p.v_bs + kvh * p.v_hs);
+    c1rs = (uint32_t)(p.k_rs * 2);
+    c2rs = (uint32_t)(p.v_rs * 2);
+  } else {
+    c1base = reinterpret_cast<const char*>(p.q + batch * p.q_bs + kvh * p.ratio * p.q_hs);
+    c2base = reinterpret_cast<const char*>(p.dout + batch * p.do_bs + kvh * p.ratio * p.do_hs);
+    c1rs = (uint32_t)(p.q_rs * 2);
+    c2rs = (uint32_t)(p.do_rs * 2);
+    c1hs = p.q_hs * 2;
+    c2hs = p.do_hs * 2;
+  }
+  auto col_pos = [&](int c) { return ROWS_ARE_QUERIES ? map.kpos(c) : map.qpos(c); };
+  auto load_tile = [&](const Cursor& cu, int slot_off) {
 #pragma unroll
-      for (int gi = 0; gi < 2; ++gi) {
-        const int grp = wave * 2 + gi;
-        const int c = im_min(cb + tile * BN + 4 * grp + ld_row, n_cols - 1);
-        const uint32_t pos = col_pos(c);
-        dma_group(c1base + ((uint64_t)pos * c1rs + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
-        dma_group(c2base + ((uint64_t)pos * c2rs + ld_col), lds_base + slot_off + TILE_BYTES + grp * GROUP_STRIDE);
-      }
-    };
-    // column scalars of a tile (dK / dV): wavefront 0 fetches lse * log2(e) and D of its 64 columns
-    float sc_l = 0.f, sc_d = 0.f;
-    auto fetch_scalars = [&](int tile) {
-      if (!ROWS_ARE_QUERIES && wave == 0) {
-        const int c = im_min(cb + tile * BN + lane, n_cols - 1);
-        const int64_t pos = col_pos(c);
-        sc_l = p.lse[batch * p.lse_bs + hcol * p.lse_hs + pos * p.lse_ts] * 1.4426950408889634f;
-        if (MODE == BWD_DK) sc_d = p.dsum[batch * p.ds_bs + hcol * p.ds_hs + pos];
-      }
-    };
-    auto put_scalars = [&](int slot_off) {
-      if (!ROWS_ARE_QUERIES && wave == 0) {
-        float* sc = reinterpret_cast<float*>(smem + slot_off + 2 * TILE_BYTES);
-        sc[lane] = sc_l;
-        sc[64 + lane] = sc_d;
-      }
-    };
+    for (int gi = 0; gi < 2; ++gi) {
+      const int grp = wave * 2 + gi;
+      const int c = im_min(cb + cu.tile * BN + 4 * grp + ld_row, n_cols - 1);
+      const uint32_t pos = col_pos(c);
+      dma_group(c1base + (cu.head * c1hs + (uint64_t)pos * c1rs + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
+      dma_group(c2base + (cu.head * c2hs + (uint64_t)pos * c2rs + ld_col),
+                lds_base + slot_off + TILE_BYTES + grp * GROUP_STRIDE);
+    }
+  };
+  // column scalars of a step (dK / dV): wavefront 0 fetches lse * log2(e) and D of its 64 columns
+  float sc_l = 0.f, sc_d = 0.f;
+  auto fetch_scalars = [&](const Cursor& cu) {
+    if (!ROWS_ARE_QUERIES && wave == 0) {
+      const int c = im_min(cb + cu.tile * BN + lane, n_cols - 1);
+      const int64_t pos = col_pos(c);
+      const int hcol = kvh * p.ratio + cu.head;
+      sc_l = p.lse[batch * p.lse_bs + hcol * p.lse_hs + pos * p.lse_ts] * 1.4426950408889634f;
+      if (MODE == BWD_DK) sc_d = p.dsum[batch * p.ds_bs + hcol * p.ds_hs + pos];
+    }
+  };
+  auto put_scalars = [&](int slot_off) {
+    if (!ROWS_ARE_QUERIES && wave == 0) {
+      float* sc = reinterpret_cast<float*>(smem + slot_off + 2 * TILE_BYTES);
+      sc[lane] = sc_l;
+      sc[64 + lane] = sc_d;
+    }
+  };
+  auto zero16 = [] {
+    floatx16 z;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) z[e] = 0.f;
+    return z;
+  };
+  auto scores = [&](int off) {
+    floatx16 s = zero16();
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kread(off, ks), r1f[ks], s, 0, 0, 0);
+    return s;
+  };
 
-    __syncthreads();  // the previous stream's last tile is no longer read
-    if (ntiles > 0) {
-      load_tile(0, 0);
-      fetch_scalars(0);
-      put_scalars(0);
+  // Three tile slots: while step t works on its tile, the tile of step t+1 has landed (the scores
+  // of its first block are formed at the end of step t) and the tile of step t+2 is in flight.
+  Cursor cur{ROWS_ARE_QUERIES ? 0 : ntiles - 1, 0};  // step being computed
+  Cursor ld = cur;                                   // step being requested
+  for (int t = 0; t < 2 && t < n_steps; ++t) {
+    load_tile(ld, t * BWD_SLOT);
+    fetch_scalars(ld);
+    put_scalars(t * BWD_SLOT);
+    advance(ld);
+  }
+  int slot0 = 0, slot1 = BWD_SLOT, slot2 = 2 * BWD_SLOT;
+  floatx16 s_cur;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) s_cur[e] = 0.f;
+  bool have = false;  // s_cur and fr hold what a previous block prepared for the one that comes next
+  constexpr int NSLOT = MODE == BWD_DV ? 16 : 24;  // MFMAs per block
+  constexpr int LA = MODE == BWD_DK ? 4 : MODE == BWD_DV ? 8 : 6;  // slots between the request of an LDS operand and its use
+  static_assert(NSLOT % LA == 0, "a block must leave the ring where the next block expects it");
+  constexpr int W0 = MODE == BWD_DV ? 2 : 10;      // slot of the first weight stage
+  bf16x8 fr[LA];
+#pragma unroll
+  for (int i = 0; i < LA; ++i) fr[i] = bf16x8{};
+  for (int t = 0; t < n_steps; ++t) {
+    tile_barrier<0>();  // the tiles of steps t and t+1 have landed for everybody; nobody reads that of t-1
+    if (t + 2 < n_steps) {
+      load_tile(ld, slot2);
+      fetch_scalars(ld);
+      advance(ld);
     }
-    for (int i = 0; i < ntiles; ++i) {
-      const int slot = (i & 1) * BWD_SLOT;
-      tile_barrier<0>();  // tile i has landed for everybody; nobody reads tile i-1 any more
-      if (i + 1 < ntiles) {
-        load_tile(i + 1, BWD_SLOT - slot);
-        fetch_scalars(i + 1);
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const int jb = 2 * cur.tile + blk;
+      if (jb < jb_lo || jb > jb_hi) {
+        have = false;
+        continue;
       }
-#pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
-        const int sb_lo = cb + i * BN + 32 * blk;  // first column of the block
-        if (!wave_active || !block_wanted(wb, kpre, sb_lo)) continue;
-        const bool masked = !block_unmasked(wb, kpre, sb_lo);
-        const int c1off = slot + blk * BLOCK32, c2off = slot + TILE_BYTES + blk * BLOCK32;
-        floatx16 s, dp;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = dp[e] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kread(c1off, ks), r1f[ks], s, 0, 0, 0);
-        if (MODE != BWD_DV) {
-#pragma unroll
-          for (int ks = 0; ks < 8; ++ks)
-            dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kread(c2off, ks), r2f[ks], dp, 0, 0, 0);
+      const int sb_lo = cb + 32 * jb;  // first column of the block
+      const bool masked = !block_unmasked(wb, kpre, sb_lo);
+      // this block, the one that follows in this order, and the one after that
+      const int c1off = slot0 + blk * BLOCK32, c2off = c1off + TILE_BYTES;
+      const int c1n = blk == 0 ? c1off + BLOCK32 : slot1, c2n = c1n + TILE_BYTES;
+      const int c1nn = blk == 0 ? slot1 : slot1 + BLOCK32;
+      // Hand-scheduled: one slot is one MFMA.  dQ / dK: slots 0-7 dP of this block, 8-15 the
+      // scores of the next block, 16-23 the accumulation; dV: 0-7 scores of the next block, 8-15
+      // the accumulation.  The LDS operand of slot i is requested in slot i - LA into a ring of
+      // LA fragments, across block and step boundaries (both following blocks have landed); the
+      // weights of element pair u are formed in slot W0 + u, after dP has drained and before the
+      // accumulation needs them.  sched_barrier keeps the compiler from regrouping the slots.
+      auto fetch = [&](int i) {
+        if (MODE == BWD_DV) {
+          if (i < 8) return kread(c1n, i);
+          if (i < 16) return vread(c2off, i - 8);
+          return kread(c1nn, i - 16);
         }
-        // weights: P = exp2(s * c2 - lse2) for visible pairs, dS = P * (dP - D)
-        const float* sc = reinterpret_cast<const float*>(smem + slot + 2 * TILE_BYTES) + 32 * blk + 4 * h32;
-        bf16x8 wp[2];
+        if (i < 8) return kread(c2off, i);
+        if (i < 16) return kread(c1n, i - 8);
+        if (i < 24) return vread(c1off, i - 16);
+        return kread(c2n, i - 24);
+      };
+      if (!have) {  // first block of a run: nothing was prepared by a previous block
+        s_cur = scores(c1off);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          floatx4 l4 = {L2_row, L2_row, L2_row, L2_row}, d4 = {D_row, D_row, D_row, D_row};
-          if (!ROWS_ARE_QUERIES) {
-            l4 = *reinterpret_cast<const floatx4*>(sc + 8 * t);
-            if (MODE == BWD_DK) d4 = *reinterpret_cast<const floatx4*>(sc + 64 + 8 * t);
-          }
-          float w[4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) {
-            const int e = 4 * t + u;
-            const int col = sb_lo + 8 * t + 4 * h32 + u;
-            float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], c2, -l4[u]));
-            if (masked && !key_visible(col, kpre, lo_l, hi_l)) x = 0.f;
-            if (MODE != BWD_DV) x *= dp[e] - d4[u];
-            w[u] = x;
-          }
-          floatx2 f0 = {w[0], w[1]}, f1 = {w[2], w[3]};
-          bf16x2 h0 = __builtin_convertvector(f0, bf16x2), h1 = __builtin_convertvector(f1, bf16x2);
-          wp[t >> 1][4 * (t & 1) + 0] = h0[0];
-          wp[t >> 1][4 * (t & 1) + 1] = h0[1];
-          wp[t >> 1][4 * (t & 1) + 2] = h1[0];
-          wp[t >> 1][4 * (t & 1) + 3] = h1[1];
-        }
-        const int xoff = MODE == BWD_DV ? c2off : c1off;
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-          acc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vread(xoff, j), wp[j >> 2], acc[j & 3], 0, 0, 0);
+        for (int i = 0; i < LA; ++i) fr[i] = fetch(i);
       }
-      if (i + 1 < ntiles) put_scalars(BWD_SLOT - slot);
+      const float* sc = reinterpret_cast<const float*>(smem + slot0 + 2 * TILE_BYTES) + 32 * blk + 4 * h32;
+      if (masked) {  // scores of invisible pairs become -inf (for a positive scale): weight 0
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          if (!key_visible(sb_lo + 8 * (e >> 2) + 4 * h32 + (e & 3), kpre, lo_l, hi_l)) s_cur[e] = s_hidden;
+      }
+      floatx16 dp, s_next;
+      bf16x8 wp[2];
+      floatx4 l4[4], d4[4];
+      auto stage = [&](int u) {  // weights of elements 2u, 2u+1: P, or dS = P * (dP - D)
+        float w[2];
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+          const int e = 2 * u + v;
+          const float l = ROWS_ARE_QUERIES ? L2_row : l4[e >> 2][e & 3];
+          float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e], c2, -l));
+          if (MODE != BWD_DV) x *= dp[e] - (ROWS_ARE_QUERIES ? D_row : d4[e >> 2][e & 3]);
+          w[v] = x;
+        }
+        floatx2 f = {w[0], w[1]};
+        bf16x2 h = __builtin_convertvector(f, bf16x2);
+        wp[u >> 2][2 * (u & 3)] = h[0];
+        wp[u >> 2][2 * (u & 3) + 1] = h[1];
+      };
+#pragma unroll
+      for (int i = 0; i < NSLOT; ++i) {
+        const bf16x8 a = fr[i % LA];
+        if (MODE == BWD_DV) {
+          if (i < 8) s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, r1f[i], i == 0 ? zero16() : s_next, 0, 0, 0);
+          else acc[(i - 8) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, wp[(i - 8) >> 2], acc[(i - 8) & 3], 0, 0, 0);
+        } else {
+          if (i < 8) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, r2f[i], i == 0 ? zero16() : dp, 0, 0, 0);
+          else if (i < 16) s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, r1f[i - 8], i == 8 ? zero16() : s_next, 0, 0, 0);
+          else acc[(i - 16) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, wp[(i - 16) >> 2], acc[(i - 16) & 3], 0, 0, 0);
+        }
+        fr[i % LA] = fetch(i + LA);
+        if (!ROWS_ARE_QUERIES && i >= W0 - 2 && i < W0 + 6 && ((i - (W0 - 2)) & 1) == 0) {
+          const int t4 = (i - (W0 - 2)) >> 1;  // column scalars of elements 4*t4 .. 4*t4+3, two slots ahead
+          l4[t4] = *reinterpret_cast<const floatx4*>(sc + 8 * t4);
+          if (MODE == BWD_DK) d4[t4] = *reinterpret_cast<const floatx4*>(sc + 64 + 8 * t4);
+        }
+        if (i >= W0 && i < W0 + 8) stage(i - W0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      s_cur = s_next;
+      have = true;
     }
+    if (t + 2 < n_steps) put_scalars(slot2);
+    advance(cur);
+    const int ts = slot0;
+    slot0 = slot1;
+    slot1 = slot2;
+    slot2 = ts;
   }
 
   // ---------------------------------------------------------------- scale, round, store
