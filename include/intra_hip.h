@@ -111,10 +111,12 @@ int intra_version(void);
  *   o, lse:    output and log-sum-exp of the forward call with the same arguments
  *   dout:      gradient of o, bf16, shaped like q
  *   dq/dk/dv:  results, bf16, shaped like q / k / v (every element is written)
- *   workspace: B * H * S floats of device memory owned by the caller (holds rowsum(dout * o));
- *              contents on entry do not matter
- * Patterns: 0, 1, 4 and INTRA_LLM_BLOCK_SCATTER with offset = 0 and n_sink = 0; others return
- * INTRA_ERR_UNSUPPORTED.  Three launches on hip_stream (dq, then dk, then dv); nothing is
+ *   workspace: intra_llm_bwd_workspace(...) floats of device memory owned by the caller, 16-byte
+ *              aligned (rowsum(dout * o), and the partial sums of the sink keys); contents on
+ *              entry do not matter
+ * Patterns: all five of intra_llm_fwd_ex; INTRA_LLM_BLOCK_SCATTER with offset != 0 needs
+ * block % 256 == 0, softmax_scale must not be 0; otherwise INTRA_ERR_UNSUPPORTED.  Launches on
+ * hip_stream: dq, dk, dv, and with sinks four more for the sink rows of dk and dv; nothing is
  * allocated.  Accuracy: weights are rounded to bf16 before the second product, as in the forward
  * pass, accumulation is fp32. */
 int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse,
@@ -125,6 +127,11 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
                   const int64_t dk_strides[3], const int64_t dv_strides[3],
                   const int64_t lse_strides[3], int pattern, int group_num, int window, int block,
                   int offset, int n_sink, float softmax_scale, void* hip_stream);
+/* Floats of workspace that intra_llm_bwd needs for such a call (B*H*S rounded up to 4, plus
+ * ceil(S/1024) * B * Hkv * min(n_sink, S) * 128 with sinks); -1 if the request is invalid or
+ * unsupported (intra_last_error() says why).  No counterpart in the reference. */
+int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int group_num,
+                                int window, int block, int offset, int n_sink);
 
 /* ------------------------------------------------------------------ host-only helpers (no GPU)
  * How a call would be launched; mirrors the grid / per-set length derivation of the reference
@@ -160,6 +167,11 @@ int intra_plan_llm_ex(int pattern, int B, int S, int H, int Hkv, int group_num, 
                       int block, int offset, int n_sink, IntraPlan* plan);
 int intra_model_mask_llm_ex(int pattern, int S, int group_num, int window, int block, int offset,
                             int n_sink, int heads_per_block, uint8_t* count);
+/* The same for the dk / dv launches of intra_llm_bwd: count[q * S + k] += 1 for every (query, key)
+ * pair that the key-row decomposition (inverse index maps, sink pass) multiplies; must equal the
+ * dense mask. */
+int intra_model_mask_llm_bwd(int pattern, int S, int group_num, int window, int block, int offset,
+                             int n_sink, uint8_t* count);
 
 #ifdef __cplusplus
 }

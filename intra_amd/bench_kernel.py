@@ -114,6 +114,13 @@ def bench_llm(args):
             if S % 64 == 0:
                 cases.append(("gather1_g8", "gather1", dict(group_num=8), pairs(0, 1, B, S, H, Hkv, 8, 576)))
             cases.append(("window576", "window", dict(window=576), pairs(0, 4, B, S, H, Hkv, 8, 576)))
+            if args.model_patterns:
+                for off in (0, 1):
+                    cases.append((f"block_scatter_g2_b256_off{off}_sink64", "block_scatter",
+                                  dict(group_num=2, block=256, offset=off, n_sink=64),
+                                  pairs_ex(8, B, S, H, Hkv, 2, 575, 256, off, 64)))
+                cases.append(("window575_sink64", "window_sink", dict(window=575, n_sink=64),
+                              pairs_ex(9, B, S, H, Hkv, 2, 575, 256, 0, 64)))
             for key, pattern, kw, npairs in cases:
                 out, lse = intra_llm_attn(q, k, v, pattern, return_lse=True, **kw)
                 ms = median_ms(lambda: intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern, **kw), args.warmup, args.iters)

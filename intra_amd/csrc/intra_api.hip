@@ -386,10 +386,10 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
 
 
 // ------------------------------------------------------------------------------------ backward
-template <class MAP, int MODE, int HP>
+template <class RMAP, int MODE, int HP, bool PARTIAL = false>
 int launch_bwd(const intra::BParams& p, int64_t grid, hipStream_t stream) {
   if (grid <= 0 || grid > 0x7fffffff) return fail(INTRA_ERR_UNSUPPORTED, "backward needs more than 2^31 workgroups");
-  hipLaunchKernelGGL((intra::intra_bwd_kernel<MAP, MODE, HP>), dim3((unsigned)grid), dim3(512), 0, stream, p);
+  hipLaunchKernelGGL((intra::intra_bwd_kernel<RMAP, MODE, HP, PARTIAL>), dim3((unsigned)grid), dim3(512), 0, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
   return INTRA_OK;
@@ -405,27 +405,74 @@ int64_t bwd_grid(intra::BParams& p, int64_t pairs) {
   return 8 * bundles * p.bundle * p.items_per_pair;
 }
 
+// dQ of a forward map: row blocks of 256 / hp queries of hp heads; also writes D = rowsum(dO o O)
 template <class MAP>
-int run_bwd_map(intra::BParams p, int hp, const Request& r, hipStream_t stream) {
-  const int64_t pairs = (int64_t)MAP::num_sets(p.geom) * r.B * r.Hkv;
-  const int max_rows = MAP::max_nq(p.geom);  // these maps number queries and keys alike: nq == nk
-  // dQ: row blocks of 256 / hp queries of hp heads; writes D = rowsum(dO o O) for the dK launch
-  p.hgroups = (r.H / r.Hkv) / hp;
-  p.n_rblocks = (max_rows + 256 / hp - 1) / (256 / hp);
-  int64_t grid = bwd_grid(p, pairs);
-  int rc;
+int run_bwd_dq(intra::BParams p, int hp, hipStream_t stream) {
+  using R = intra::QueryRows<MAP>;
+  const int64_t pairs = (int64_t)R::num_sets(p.geom) * p.B * p.Hkv;
+  p.hgroups = p.ratio / hp;
+  p.n_rblocks = (R::max_rows(p.geom) + 256 / hp - 1) / (256 / hp);
+  const int64_t grid = bwd_grid(p, pairs);
   switch (hp) {
-    case 4: rc = launch_bwd<MAP, intra::BWD_DQ, 4>(p, grid, stream); break;
-    case 2: rc = launch_bwd<MAP, intra::BWD_DQ, 2>(p, grid, stream); break;
-    default: rc = launch_bwd<MAP, intra::BWD_DQ, 1>(p, grid, stream); break;
+    case 4: return launch_bwd<R, intra::BWD_DQ, 4>(p, grid, stream);
+    case 2: return launch_bwd<R, intra::BWD_DQ, 2>(p, grid, stream);
+    default: return launch_bwd<R, intra::BWD_DQ, 1>(p, grid, stream);
   }
-  if (rc) return rc;
-  // dK, dV: row blocks of 256 keys of one kv head, all query heads of its group streamed past
+}
+
+// dK then dV over a key-row map: row blocks of 256 keys of one kv head, all query heads of its
+// group streamed past
+template <class R, bool PARTIAL, int MODE>
+int run_bwd_keys_mode(intra::BParams p, hipStream_t stream) {
+  const int64_t pairs = (int64_t)R::num_sets(p.geom) * p.B * p.Hkv;
   p.hgroups = 1;
-  p.n_rblocks = (max_rows + 255) / 256;
-  grid = bwd_grid(p, pairs);
-  if ((rc = launch_bwd<MAP, intra::BWD_DK, 1>(p, grid, stream))) return rc;
-  return launch_bwd<MAP, intra::BWD_DV, 1>(p, grid, stream);
+  p.n_rblocks = (R::max_rows(p.geom) + 255) / 256;
+  return launch_bwd<R, MODE, 1, PARTIAL>(p, bwd_grid(p, pairs), stream);
+}
+template <class R>
+int run_bwd_keys(const intra::BParams& p, hipStream_t stream) {
+  if (int rc = run_bwd_keys_mode<R, false, intra::BWD_DK>(p, stream)) return rc;
+  return run_bwd_keys_mode<R, false, intra::BWD_DV>(p, stream);
+}
+
+// The sink rows of dk and dv: partial sums per chunk of queries, then their sum (twice, dk and dv
+// share the partial buffer; everything is ordered by the stream).
+int run_bwd_sinks(const intra::BParams& p, hipStream_t stream) {
+  using R = intra::KeyRowsSinks;
+  const int ns = R::max_rows(p.geom), chunks = R::num_sets(p.geom);
+  const int64_t threads = (int64_t)p.B * p.Hkv * ns * 32;
+  const unsigned blocks = (unsigned)((threads + 255) / 256);
+  for (int mode = 0; mode < 2; ++mode) {
+    int rc = mode == 0 ? run_bwd_keys_mode<R, true, intra::BWD_DK>(p, stream)
+                       : run_bwd_keys_mode<R, true, intra::BWD_DV>(p, stream);
+    if (rc) return rc;
+    if (mode == 0)
+      hipLaunchKernelGGL(intra::intra_bwd_sink_reduce, dim3(blocks), dim3(256), 0, stream, p.part, chunks, p.B, p.Hkv,
+                         ns, p.dk, p.dk_bs, p.dk_rs, p.dk_hs);
+    else
+      hipLaunchKernelGGL(intra::intra_bwd_sink_reduce, dim3(blocks), dim3(256), 0, stream, p.part, chunks, p.B, p.Hkv,
+                         ns, p.dv, p.dv_bs, p.dv_rs, p.dv_hs);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+  }
+  return INTRA_OK;
+}
+
+// floats of workspace: D = rowsum(dO o O) per (batch, head, token), then the partial sums of the sink pass
+int64_t bwd_dsum_floats(int B, int S, int H) { return ((int64_t)B * H * S + 3) & ~(int64_t)3; }
+int64_t bwd_workspace_floats(const Request& r) {
+  int64_t n = bwd_dsum_floats(r.B, r.S, r.H);
+  const int ns = std::min(r.geom.ns, r.S);
+  if ((r.kind == KIND_LLM_BLOCK_SCATTER || r.kind == KIND_LLM_WINDOW_SINK) && ns > 0)
+    n += (int64_t)((r.S + intra::SINK_CHUNK - 1) / intra::SINK_CHUNK) * r.B * r.Hkv * ns * 128;
+  return n;
+}
+
+// Does the backward pass cover this request?
+int bwd_supported(const Request& r) {
+  if (r.kind == KIND_LLM_BLOCK_SCATTER && r.geom.off != 0 && r.geom.blk % 256 != 0)
+    return fail(INTRA_ERR_UNSUPPORTED, "backward: block scatter with a stripe offset needs block % 256 == 0");
+  return INTRA_OK;
 }
 
 int run_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
@@ -437,16 +484,14 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
   Request r;
   int rc = make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true);
   if (rc) return rc;
-  if (r.kind == KIND_LLM_WINDOW_SINK || (r.kind == KIND_LLM_BLOCK_SCATTER && (offset != 0 || n_sink != 0)))
-    return fail(INTRA_ERR_UNSUPPORTED,
-                "backward: dK / dV are built for scatter, gather1, window and block scatter without offset and sinks");
+  if ((rc = bwd_supported(r))) return rc;
   const void* ins[] = {q, k, v, o, dout, dq, dk, dv};
   for (const void* ptr : ins) {
     if (!ptr) return fail(INTRA_ERR_INVALID, "q, k, v, o, dout, dq, dk and dv must be non-null device pointers");
     if (!aligned16(ptr)) return fail(INTRA_ERR_INVALID, "q, k, v, o, dout, dq, dk and dv must be 16-byte aligned");
   }
-  if (!lse || !dsum || (reinterpret_cast<uintptr_t>(lse) & 3) || (reinterpret_cast<uintptr_t>(dsum) & 3))
-    return fail(INTRA_ERR_INVALID, "lse and the workspace must be non-null, 4-byte aligned device pointers");
+  if (!lse || (reinterpret_cast<uintptr_t>(lse) & 3)) return fail(INTRA_ERR_INVALID, "lse must be a non-null, 4-byte aligned device pointer");
+  if (!dsum || !aligned16(dsum)) return fail(INTRA_ERR_INVALID, "the workspace must be a non-null, 16-byte aligned device pointer");
   if ((rc = check_strides("q", qs, B, S, H)) || (rc = check_strides("k", ks, B, S, Hkv)) ||
       (rc = check_strides("v", vs, B, S, Hkv)) || (rc = check_strides("o", os, B, S, H)) ||
       (rc = check_strides("dout", dos, B, S, H)) || (rc = check_strides("odq", dqs, B, S, H)) ||
@@ -467,6 +512,7 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
   p.dout = static_cast<const uint16_t*>(dout);
   p.lse = lse;
   p.dsum = dsum;
+  p.part = dsum + bwd_dsum_floats(B, S, H);
   p.dq = static_cast<uint16_t*>(dq);
   p.dk = static_cast<uint16_t*>(dk);
   p.dv = static_cast<uint16_t*>(dv);
@@ -488,11 +534,62 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
   p.geom = sh.geom;
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (sh.map) {
-    case MAP_LLM_SCATTER: return run_bwd_map<MapLlmScatter>(p, sh.hp, r, st);
-    case MAP_LLM_GATHER1: return run_bwd_map<MapLlmGather1>(p, sh.hp, r, st);
-    case MAP_LLM_WINDOW: return run_bwd_map<MapLlmWindow>(p, sh.hp, r, st);
-    default: return run_bwd_map<MapLlmBlockScatter>(p, sh.hp, r, st);
+    case MAP_LLM_SCATTER:
+      if ((rc = run_bwd_dq<MapLlmScatter>(p, sh.hp, st))) return rc;
+      return run_bwd_keys<intra::KeyRowsOf<MapLlmScatter>>(p, st);
+    case MAP_LLM_GATHER1:
+      if ((rc = run_bwd_dq<MapLlmGather1>(p, sh.hp, st))) return rc;
+      return run_bwd_keys<intra::KeyRowsOf<MapLlmGather1>>(p, st);
+    case MAP_LLM_WINDOW:
+      if ((rc = run_bwd_dq<MapLlmWindow>(p, sh.hp, st))) return rc;
+      return run_bwd_keys<intra::KeyRowsOf<MapLlmWindow>>(p, st);
+    case MAP_LLM_BLOCK_SCATTER:
+      if ((rc = run_bwd_dq<MapLlmBlockScatter>(p, sh.hp, st))) return rc;
+      if ((rc = run_bwd_keys<intra::KeyRowsBlockScatter>(p, st))) return rc;
+      break;
+    case MAP_LLM_WINDOW_SINK:
+      if ((rc = run_bwd_dq<MapLlmWindowSink>(p, sh.hp, st))) return rc;
+      if ((rc = run_bwd_keys<intra::KeyRowsWindowSink>(p, st))) return rc;
+      break;
+    default: return fail(INTRA_ERR_UNSUPPORTED, "backward: no kernels for this pattern");
   }
+  return std::min(r.geom.ns, r.S) > 0 ? run_bwd_sinks(p, st) : INTRA_OK;
+}
+
+// Host walk of the backward decomposition: count[q * S + k] += 1 for every (query, key) pair that
+// the dK / dV launches (key-row maps with their `store` rule, then the sink pass) multiply.
+template <class R>
+void bwd_walk(const IntraGeom& ge, uint8_t* count) {
+  const int S = ge.S;
+  for (int set = 0; set < R::num_sets(ge); ++set)
+    for (int r0 = 0; r0 < R::max_rows(ge); r0 += 256) {
+      const R m(ge, set, r0);
+      const int r1 = std::min(r0 + 256, m.n_rows()) - 1;
+      for (int t = r0; t <= r1; ++t) {
+        const int kp = m.row_pos(t);
+        if (!m.store(kp)) continue;
+        const int lo = m.lo(t), hi = std::min(m.hi(t), m.n_cols() - 1);
+        for (int c = std::max(lo, m.block_lo(r0, r1)); c <= std::min(hi, m.block_hi(r0, r1)); ++c)
+          ++count[(size_t)m.col_pos(c) * S + kp];
+      }
+    }
+}
+
+int model_mask_bwd(const Request& r, uint8_t* count) {
+  if (int rc = bwd_supported(r)) return rc;
+  Shape sh;
+  if (!shape_for(r, 1, &sh)) return fail(INTRA_ERR_UNSUPPORTED, "no kernel shape for this request");
+  switch (sh.map) {
+    case MAP_LLM_SCATTER: bwd_walk<intra::KeyRowsOf<MapLlmScatter>>(sh.geom, count); break;
+    case MAP_LLM_GATHER1: bwd_walk<intra::KeyRowsOf<MapLlmGather1>>(sh.geom, count); break;
+    case MAP_LLM_WINDOW: bwd_walk<intra::KeyRowsOf<MapLlmWindow>>(sh.geom, count); break;
+    case MAP_LLM_BLOCK_SCATTER: bwd_walk<intra::KeyRowsBlockScatter>(sh.geom, count); break;
+    case MAP_LLM_WINDOW_SINK: bwd_walk<intra::KeyRowsWindowSink>(sh.geom, count); break;
+    default: return fail(INTRA_ERR_UNSUPPORTED, "backward: no kernels for this pattern");
+  }
+  if (std::min(r.geom.ns, r.S) > 0 && (sh.map == MAP_LLM_BLOCK_SCATTER || sh.map == MAP_LLM_WINDOW_SINK))
+    bwd_walk<intra::KeyRowsSinks>(sh.geom, count);
+  return INTRA_OK;
 }
 
 int model_mask(const Request& r, int heads_per_block, int waves, uint8_t* count) {
@@ -554,6 +651,25 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
   return run_bwd(q, k, v, o, lse, dout, dq, dk, dv, workspace, B, S, H, Hkv, q_strides, k_strides, v_strides,
                  o_strides, dout_strides, dq_strides, dk_strides, dv_strides, lse_strides, pattern, group_num,
                  window, block, offset, n_sink, softmax_scale, hip_stream);
+}
+
+int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int group_num, int window, int block,
+                                int offset, int n_sink) {
+  g_err[0] = 0;
+  Request r;
+  if (make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true)) return -1;
+  if (bwd_supported(r)) return -1;
+  return bwd_workspace_floats(r);
+}
+
+int intra_model_mask_llm_bwd(int pattern, int S, int group_num, int window, int block, int offset, int n_sink,
+                             uint8_t* count) {
+  g_err[0] = 0;
+  if (!count) return fail(INTRA_ERR_INVALID, "count is null");
+  Request r;
+  int rc = make_request(0, pattern, 1, S, 1, 1, group_num, window, &r, block, offset, n_sink, true);
+  if (rc) return rc;
+  return model_mask_bwd(r, count);
 }
 
 const char* intra_last_error(void) { return g_err; }

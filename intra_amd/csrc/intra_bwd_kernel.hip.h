@@ -18,6 +18,7 @@
 // index maps; for dK / dV the query range of a key is found by bisection on the maps' monotone
 // bounds, so no pattern needs inverse formulas.
 #pragma once
+#include "intra_bwd_maps.h"
 #include "intra_kernel.hip.h"
 
 namespace intra {
@@ -31,6 +32,7 @@ struct BParams {
   const float* lse;                      // (B, H, S): ln sum exp(scale * q.k) from the forward pass
   float* dsum;                           // (B, H, S) workspace: D = rowsum(dO o O), written by dQ, read by dK
   uint16_t *dq, *dk, *dv;
+  float* part;  // partial sums of the sink pass: (chunk, batch, kv head, sink, 128) fp32
   // element strides: batch, row (token), head
   int64_t q_bs, q_rs, q_hs, k_bs, k_rs, k_hs, v_bs, v_rs, v_hs, o_bs, o_rs, o_hs, do_bs, do_rs, do_hs;
   int64_t dq_bs, dq_rs, dq_hs, dk_bs, dk_rs, dk_hs, dv_bs, dv_rs, dv_hs;
@@ -48,12 +50,13 @@ struct BParams {
 constexpr int BWD_SLOT = 2 * TILE_BYTES + 512;  // two tiles and 2 x 64 column scalars
 constexpr int BWD_LDS_BYTES = 3 * BWD_SLOT;
 
-template <class MAP, int MODE, int HP>
+// RMAP: row map (intra_bwd_maps.h).  PARTIAL: the results are partial sums over the set's columns,
+// written as fp32 to p.part instead of bf16 to dk / dv (sink pass).
+template <class RMAP, int MODE, int HP, bool PARTIAL = false>
 __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   constexpr int NW = 8;
   constexpr bool ROWS_ARE_QUERIES = MODE == BWD_DQ;
   constexpr int POS = ROWS_ARE_QUERIES ? NW * 32 / HP : NW * 32;  // rows per row block (of one head)
-  static_assert(!MAP::kHasPrefix, "built for maps whose rows meet one contiguous range of columns");
 
   __shared__ __attribute__((aligned(1024))) unsigned char smem[BWD_LDS_BYTES];
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   const int heavy = rem / p.bundle;
   const int nbh = p.B * p.Hkv;
   const int pair = (bun * p.bundle + (rem - heavy * p.bundle)) * 8 + xcd;
-  if (pair >= MAP::num_sets(p.geom) * nbh) return;
+  if (pair >= RMAP::num_sets(p.geom) * nbh) return;
   int hg = 0, rblk = heavy;
   if (ROWS_ARE_QUERIES) {
     hg = heavy % p.hgroups;
@@ -88,58 +91,46 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   const int kvh = bh % p.Hkv;
 
   const int r0 = rblk * POS;
-  const MAP map(p.geom, set, ROWS_ARE_QUERIES ? r0 : 0);
-  const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
-  const int n_rows = ROWS_ARE_QUERIES ? nq : nk;
-  const int n_cols = ROWS_ARE_QUERIES ? nk : nq;
+  const RMAP map(p.geom, set, r0);
+  const int kpre = map.kpre();
+  const int n_rows = map.n_rows(), n_cols = map.n_cols();
   if (r0 >= n_rows) return;
   const int r1 = im_min(r0 + POS, n_rows) - 1;
 
-  // Columns a row meets: [col_lo(r), col_hi(r)] (plus the prefix below kpre for maps that have one).
-  // For key rows the bounds are the first query whose upper key bound reaches the key and the last
-  // one whose lower key bound does not exceed it; both are monotone in the key.
-  auto col_lo = [&](int r) {
-    if (ROWS_ARE_QUERIES) return map.klo(r);
-    int lo = 0, hi = nq;  // first tq with min(khi(tq), nk-1) >= r
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (im_min(map.khi(mid), nk - 1) >= r) hi = mid;
-      else lo = mid + 1;
-    }
-    return lo;
-  };
-  auto col_hi = [&](int r) {
-    if (ROWS_ARE_QUERIES) return im_min(map.khi(r), nk - 1);
-    int lo = -1, hi = nq - 1;  // last tq with klo(tq) <= r
-    while (lo < hi) {
-      const int mid = (lo + hi + 1) >> 1;
-      if (map.klo(mid) <= r) lo = mid;
-      else hi = mid - 1;
-    }
-    return lo;
-  };
-
-  const int cb = col_lo(r0);  // first column of the row block
-  const int ce = col_hi(r1);                                             // last one
+  // Row r meets the columns lo(r)..hi(r) (plus those below kpre for maps that have such a prefix).
+  const int cb = map.block_lo(r0, r1);  // first column of the row block
+  const int ce = map.block_hi(r0, r1);  // last one
   const int ntiles = ce >= cb ? (ce - cb + BN) / BN : 0;
 
   // ---------------------------------------------------------------- this wavefront's rows
   const int hw = ROWS_ARE_QUERIES ? wave % HP : 0;
   const int wr0 = r0 + (ROWS_ARE_QUERIES ? wave / HP : wave) * 32;
   const bool wave_active = wr0 <= r1;
-  const int wr_last = im_min(wr0 + 31, r1);
   const bool row_valid = wr0 + l32 <= r1;
   const int row = im_min(wr0 + l32, r1);
-  const int lo_l = col_lo(row), hi_l = col_hi(row);
+  const int lo_l = map.lo(row), hi_l = map.hi(row);
+  // union and intersection of the ranges of the wavefront's rows (rows past the end repeat the last)
   WaveBounds wb;
-  wb.w_lo = __builtin_amdgcn_readfirstlane(col_lo(im_min(wr0, r1)));
-  wb.w_hi = __builtin_amdgcn_readfirstlane(col_hi(wr_last));
-  wb.f_lo = __builtin_amdgcn_readfirstlane(col_lo(wr_last));
-  wb.f_hi = __builtin_amdgcn_readfirstlane(col_hi(im_min(wr0, r1)));
-  // the blocks of 32 columns (counted from cb) that this wavefront's rows meet: one range
-  const int jb_lo = wave_active ? (wb.w_lo - cb) >> 5 : 1;
-  const int jb_hi = wave_active ? (wb.w_hi - cb) >> 5 : 0;
-  const int64_t rpos = ROWS_ARE_QUERIES ? map.qpos(row) : map.kpos(row);
+  {
+    int a = lo_l, b = hi_l, c = lo_l, d = hi_l;
+#pragma unroll
+    for (int m = 1; m < 32; m <<= 1) {
+      a = im_min(a, __shfl_xor(a, m));
+      b = im_max(b, __shfl_xor(b, m));
+      c = im_max(c, __shfl_xor(c, m));
+      d = im_min(d, __shfl_xor(d, m));
+    }
+    wb.w_lo = __builtin_amdgcn_readfirstlane(a);
+    wb.w_hi = __builtin_amdgcn_readfirstlane(b);
+    wb.f_lo = __builtin_amdgcn_readfirstlane(c);
+    wb.f_hi = __builtin_amdgcn_readfirstlane(d);
+  }
+  // The blocks of 32 columns (counted from cb) that this wavefront's rows meet: one range; with a
+  // prefix it starts at the first block (blocks between prefix and own range are few and masked).
+  const bool any = wave_active && wb.w_hi >= cb && (kpre > 0 || wb.w_hi >= wb.w_lo);  // (early rows may meet prefix columns only)
+  const int jb_lo = !any ? 1 : kpre > 0 ? 0 : (im_max(wb.w_lo, cb) - cb) >> 5;
+  const int jb_hi = !any ? 0 : (wb.w_hi - cb) >> 5;
+  const int64_t rpos = map.row_pos(row);
   const int hq = kvh * p.ratio + hg * HP + hw;  // query head of a query row
 
   // ---------------------------------------------------------------- row operands (MFMA B fragments)
@@ -242,7 +233,7 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
     c1hs = p.q_hs * 2;
     c2hs = p.do_hs * 2;
   }
-  auto col_pos = [&](int c) { return ROWS_ARE_QUERIES ? map.kpos(c) : map.qpos(c); };
+  auto col_pos = [&](int c) { return map.col_pos(c); };
   auto load_tile = [&](const Cursor& cu, int slot_off) {
 #pragma unroll
     for (int gi = 0; gi < 2; ++gi) {
@@ -407,6 +398,22 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   // ---------------------------------------------------------------- scale, round, store
   if (!wave_active) return;
   const float f = MODE == BWD_DV ? 1.f : p.scale;
+  if (PARTIAL) {
+    // fp32 partial sums: part[((set * B + batch) * Hkv + kvh) * n_rows + row][128]; lane holds, per
+    // 32 head dims db, the dims 8*(e>>2) + 4*h32 + (e&3) of its row
+    if (row_valid) {
+      float* prow = p.part + ((((int64_t)set * p.B + batch) * p.Hkv + kvh) * n_rows + row) * 128 + 4 * h32;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; ++g4) {
+          floatx4 o4 = {acc[db][4 * g4] * f, acc[db][4 * g4 + 1] * f, acc[db][4 * g4 + 2] * f, acc[db][4 * g4 + 3] * f};
+          *reinterpret_cast<floatx4*>(prow + 32 * db + 8 * g4) = o4;
+        }
+    }
+    return;
+  }
+  const bool keep = row_valid && map.store((int)rpos);
   uint16_t* orow;
   if (MODE == BWD_DQ) orow = p.dq + (batch * p.dq_bs + rpos * p.dq_rs + hq * p.dq_hs + 8 * h32);
   else if (MODE == BWD_DK) orow = p.dk + (batch * p.dk_bs + rpos * p.dk_rs + kvh * p.dk_hs + 8 * h32);
@@ -419,18 +426,39 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
 #pragma unroll
       for (int half = 0; half < 2; ++half)
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-          const int e = 8 * g2 + 4 * half + 2 * k;
+        for (int k2 = 0; k2 < 2; ++k2) {
+          const int e = 8 * g2 + 4 * half + 2 * k2;
           floatx2 v2 = {acc[db][e] * f, acc[db][e + 1] * f};
-          w[2 * half + k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
+          w[2 * half + k2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
         }
       auto q0 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
       auto q1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
-      if (row_valid) {
+      if (keep) {
         u32x4 pk = {q0[0], q1[0], q0[1], q1[1]};
         *reinterpret_cast<u32x4*>(orow + 32 * db + 16 * g2) = pk;
       }
     }
+}
+
+// Adds up the partial sums of the sink pass over the chunks and writes the sink rows of dk or dv:
+// one thread per (batch, kv head, sink, 4 head dims).
+__global__ void intra_bwd_sink_reduce(const float* part, int n_chunks, int B, int Hkv, int ns, uint16_t* out,
+                                      int64_t o_bs, int64_t o_rs, int64_t o_hs) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = (int64_t)B * Hkv * ns * 32;
+  if (i >= total) return;
+  const int d4 = (int)(i & 31);
+  const int64_t row = i >> 5;  // (batch * Hkv + kvh) * ns + sink
+  floatx4 s = {0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < n_chunks; ++c) s += *reinterpret_cast<const floatx4*>(part + ((int64_t)c * B * Hkv * ns + row) * 128 + 4 * d4);
+  const int sink = (int)(row % ns);
+  const int64_t bh = row / ns;
+  const int kvh = (int)(bh % Hkv), batch = (int)(bh / Hkv);
+  floatx2 a = {s[0], s[1]}, b = {s[2], s[3]};
+  uint32_t lo = __builtin_bit_cast(uint32_t, __builtin_convertvector(a, bf16x2));
+  uint32_t hi = __builtin_bit_cast(uint32_t, __builtin_convertvector(b, bf16x2));
+  uint16_t* o = out + (batch * o_bs + sink * o_rs + kvh * o_hs + 4 * d4);
+  *reinterpret_cast<uint2*>(o) = make_uint2(lo, hi);
 }
 
 }  // namespace intra

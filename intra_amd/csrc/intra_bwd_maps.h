@@ -1,0 +1,188 @@
+// Row maps of the backward kernels: which "columns" a block of "rows" meets.
+//
+// dQ: rows are the queries of a set and columns its keys - the forward index map as it is
+// (QueryRows).  dK / dV: rows are keys and columns the queries that see them.  For the patterns
+// whose sets number queries and keys alike, the query range of a key follows from the forward
+// map's monotone bounds by bisection (KeyRowsOf).  Block Scatter with a stripe offset and the
+// per-token window have their own inverse maps.  Keys that are sinks are seen by every later
+// query of every set; they are left out of those maps' results (`store`) and get a pass of their
+// own (KeyRowsSinks), split over chunks of queries whose partial sums a small kernel adds up.
+//
+// Interface (host and device):
+//   static num_sets(ge), max_rows(ge)      grid size: sets per (batch, kv head), rows of the largest
+//   RowMap(ge, set, r0)                    r0: first row of the row block (rows r0 .. r0+255 at most)
+//   n_rows(), n_cols()
+//   row_pos(t), col_pos(c)                 token positions
+//   lo(t), hi(t)                           row t meets the columns lo..hi (and those below kpre())
+//   block_lo(r0, r1), block_hi(r0, r1)     union of the ranges of rows r0..r1
+//   store(pos)                             whether the result row of token pos is written here
+#pragma once
+#include "intra_maps.h"
+
+namespace intra {
+
+constexpr int SINK_CHUNK = 1024;  // queries per workgroup of the sink pass
+
+template <class MAP>
+struct QueryRows {
+  MAP m;
+  static IM_HD int num_sets(const IntraGeom& ge) { return MAP::num_sets(ge); }
+  static IM_HD int max_rows(const IntraGeom& ge) { return MAP::max_nq(ge); }
+  IM_HD QueryRows(const IntraGeom& ge, int set, int r0) : m(ge, set, r0) {}
+  IM_HD int n_rows() const { return m.nq(); }
+  IM_HD int n_cols() const { return m.nk(); }
+  IM_HD int kpre() const { return m.kpre(); }
+  IM_HD int row_pos(int t) const { return m.qpos(t); }
+  IM_HD int col_pos(int c) const { return m.kpos(c); }
+  IM_HD int lo(int t) const { return m.klo(t); }
+  IM_HD int hi(int t) const { return im_min(m.khi(t), m.nk() - 1); }
+  IM_HD int block_lo(int r0, int) const { return m.kpre() > 0 ? 0 : m.klo(r0); }
+  IM_HD int block_hi(int, int r1) const { return hi(r1); }
+  IM_HD bool store(int) const { return true; }
+};
+
+// Keys of a set whose queries and keys carry the same numbering (LLM Scatter, Gather 1, window,
+// block Scatter without offset): key r is seen by the queries from the first one whose upper key
+// bound reaches r to the last one whose lower key bound does not exceed r; both are monotone in r.
+template <class MAP>
+struct KeyRowsOf {
+  MAP m;
+  int skip;
+  static IM_HD int num_sets(const IntraGeom& ge) { return MAP::num_sets(ge); }
+  static IM_HD int max_rows(const IntraGeom& ge) { return MAP::max_nq(ge); }
+  IM_HD KeyRowsOf(const IntraGeom& ge, int set, int) : m(ge, set, 0), skip(0) {}
+  IM_HD int n_rows() const { return m.nk(); }
+  IM_HD int n_cols() const { return m.nq(); }
+  IM_HD int kpre() const { return 0; }
+  IM_HD int row_pos(int t) const { return m.kpos(t); }
+  IM_HD int col_pos(int c) const { return m.qpos(c); }
+  IM_HD int lo(int r) const {  // first tq with min(khi(tq), nk-1) >= r
+    int a = 0, b = m.nq();
+    const int kmax = m.nk() - 1;
+    while (a < b) {
+      const int mid = (a + b) >> 1;
+      if (im_min(m.khi(mid), kmax) >= r) b = mid;
+      else a = mid + 1;
+    }
+    return a;
+  }
+  IM_HD int hi(int r) const {  // last tq with klo(tq) <= r
+    int a = -1, b = m.nq() - 1;
+    while (a < b) {
+      const int mid = (a + b + 1) >> 1;
+      if (m.klo(mid) <= r) a = mid;
+      else b = mid - 1;
+    }
+    return a;
+  }
+  IM_HD int block_lo(int r0, int) const { return lo(r0); }
+  IM_HD int block_hi(int, int r1) const { return hi(r1); }
+  IM_HD bool store(int) const { return true; }
+};
+
+// Keys of group gk of block Scatter (blocks kb = gk mod G), any stripe offset.  Without offset the
+// queries that see them are the later tokens of the same group.  With offset `off` a key of block
+// kb is seen by the later queries of its own block and by all queries of the blocks kb + G - off,
+// kb + 2G - off, ... (the query blocks qb > kb with (qb + off) mod G = gk); the columns of a row
+// block are numbered [own block][those blocks], which needs the row block inside one key block
+// (block size a multiple of 256).  Sinks (positions < n_sink) are not stored here.
+struct KeyRowsBlockScatter {
+  int G, blk, gk, off, n, S, skip, a, kb, own_len, qb0, ncols;
+  FastDiv dBlk;
+  static IM_HD int num_sets(const IntraGeom& ge) { return ge.G; }
+  static IM_HD int max_rows(const IntraGeom& ge) { return MapLlmBlockScatter::max_nq(ge); }
+  IM_HD KeyRowsBlockScatter(const IntraGeom& ge, int set, int r0) {
+    G = ge.G;
+    blk = ge.blk;
+    off = ge.off;
+    S = ge.S;
+    dBlk = ge.dBlk;
+    gk = set;
+    skip = im_min(ge.ns, ge.S);
+    n = MapLlmBlockScatter::group_size(ge, gk);
+    a = (int)fd_div(r0, dBlk);
+    kb = a * G + gk;
+    own_len = im_max(0, im_min(blk, S - kb * blk));
+    qb0 = kb + G - off;
+    if (off == 0) {
+      ncols = n;
+    } else {
+      const int nbt = (int)fd_div(S + blk - 1, dBlk);  // blocks in the sequence, the last one maybe short
+      int later = 0;
+      if (qb0 < nbt) {
+        const int cnt = (int)fd_div(nbt - 1 - qb0, ge.dG) + 1;  // blocks qb0, qb0 + G, ... below nbt
+        const int last = qb0 + (cnt - 1) * G;
+        later = (cnt - 1) * blk + im_min(blk, S - last * blk);
+      }
+      ncols = own_len + later;
+    }
+  }
+  IM_HD int n_rows() const { return n; }
+  IM_HD int n_cols() const { return ncols; }
+  IM_HD int kpre() const { return 0; }
+  IM_HD int row_pos(int t) const {
+    const int b = (int)fd_div(t, dBlk);
+    return (b * G + gk) * blk + (t - b * blk);
+  }
+  IM_HD int col_pos(int c) const {
+    if (off == 0) return row_pos(c);
+    if (c < own_len) return kb * blk + c;
+    const int c2 = c - own_len;
+    const int m = (int)fd_div(c2, dBlk);
+    return (qb0 + m * G) * blk + (c2 - m * blk);
+  }
+  IM_HD int lo(int t) const { return off == 0 ? t : t - a * blk; }
+  IM_HD int hi(int) const { return ncols - 1; }
+  IM_HD int block_lo(int r0, int) const { return lo(r0); }
+  IM_HD int block_hi(int, int) const { return ncols - 1; }
+  IM_HD bool store(int pos) const { return pos >= skip; }
+};
+
+// Keys of the per-token window with sinks: key j is seen by the queries j .. j + window - 1.
+// Sinks (j < n_sink; seen by every later query) are not stored here.
+struct KeyRowsWindowSink {
+  int S, window, skip;
+  static IM_HD int num_sets(const IntraGeom&) { return 1; }
+  static IM_HD int max_rows(const IntraGeom& ge) { return ge.S; }
+  IM_HD KeyRowsWindowSink(const IntraGeom& ge, int, int) {
+    S = ge.S;
+    window = ge.window;
+    skip = im_min(ge.ns, ge.S);
+  }
+  IM_HD int n_rows() const { return S; }
+  IM_HD int n_cols() const { return S; }
+  IM_HD int kpre() const { return 0; }
+  IM_HD int row_pos(int t) const { return t; }
+  IM_HD int col_pos(int c) const { return c; }
+  IM_HD int lo(int t) const { return t; }
+  IM_HD int hi(int t) const { return (int)im_min64((int64_t)t + window - 1, S - 1); }
+  IM_HD int block_lo(int r0, int) const { return r0; }
+  IM_HD int block_hi(int, int r1) const { return hi(r1); }
+  IM_HD bool store(int pos) const { return pos >= skip; }
+};
+
+// The sink keys (positions below n_sink) against every later query of the sequence; set = chunk
+// of SINK_CHUNK queries.  The results are partial sums over the chunk.
+struct KeyRowsSinks {
+  int S, ns, c0, c1;
+  static IM_HD int num_sets(const IntraGeom& ge) { return (ge.S + SINK_CHUNK - 1) / SINK_CHUNK; }
+  static IM_HD int max_rows(const IntraGeom& ge) { return im_min(ge.ns, ge.S); }
+  IM_HD KeyRowsSinks(const IntraGeom& ge, int set, int) {
+    S = ge.S;
+    ns = im_min(ge.ns, ge.S);
+    c0 = set * SINK_CHUNK;
+    c1 = im_min(c0 + SINK_CHUNK, S);
+  }
+  IM_HD int n_rows() const { return ns; }
+  IM_HD int n_cols() const { return S; }
+  IM_HD int kpre() const { return 0; }
+  IM_HD int row_pos(int t) const { return t; }
+  IM_HD int col_pos(int c) const { return c; }
+  IM_HD int lo(int t) const { return im_max(t, c0); }
+  IM_HD int hi(int) const { return c1 - 1; }
+  IM_HD int block_lo(int r0, int) const { return im_max(r0, c0); }
+  IM_HD int block_hi(int, int) const { return c1 - 1; }
+  IM_HD bool store(int) const { return true; }
+};
+
+}  // namespace intra

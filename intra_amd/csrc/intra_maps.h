@@ -100,6 +100,7 @@ inline void geom_finish(IntraGeom& ge) {
 
 IM_HD int im_min(int a, int b) { return a < b ? a : b; }
 IM_HD int im_max(int a, int b) { return a > b ? a : b; }
+IM_HD int64_t im_min64(int64_t a, int64_t b) { return a < b ? a : b; }
 
 // ---------------------------------------------------------------- LLM scatter: token i in group i % G
 struct MapLlmScatter {

@@ -127,15 +127,16 @@ def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_
 
 
 def intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", group_num=8, window=576, softmax_scale=None,
-                       block=256):
-    """Gradients (dq, dk, dv) of intra_llm_attn for pattern "scatter", "gather1", "window" or
-    "block_scatter" (offset 0, no sinks), given the forward results `out`, `lse` (return_lse=True)
-    and the gradient `dout` of `out`.  The reference has no backward kernels (its training runs
-    differentiate masked SDPA, experiments/llm/llama_intra.py:26)."""
+                       block=256, offset=0, n_sink=0):
+    """Gradients (dq, dk, dv) of intra_llm_attn for any of its patterns, given the forward results
+    `out`, `lse` (return_lse=True) and the gradient `dout` of `out`; the pattern arguments are those
+    of the forward call.  block_scatter with offset != 0 needs block % 256 == 0.  The reference has
+    no backward kernels (its training runs differentiate masked SDPA,
+    experiments/llm/llama_intra.py:26)."""
     q, k, v = _check(q, k, v)
-    ids = dict(LLM_PATTERNS, block_scatter=EXTRA_LLM_PATTERNS["block_scatter"])
+    ids = dict(LLM_PATTERNS, **EXTRA_LLM_PATTERNS)
     if pattern not in ids:
-        raise ValueError(f"no backward kernels for pattern {pattern!r}")
+        raise ValueError(f"unknown pattern {pattern!r}")
     if pattern == "gather1" and (group_num != 8 or q.shape[1] % (group_num * group_num)):
         raise ValueError(f"gather1 needs group_num=8 and seqlen % 64 == 0, got G={group_num}, S={q.shape[1]}")
     fix = lambda t: t if (t.stride(-1) == 1 and _aligned(t)) else t.contiguous()
@@ -145,16 +146,19 @@ def intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", group_num=8, 
     B, S, H, _ = q.shape
     if lse.shape != (B, H, S) or lse.dtype != torch.float32:
         raise ValueError("lse must be the (batch, heads, seqlen) fp32 tensor of the forward call")
+    args = (ids[pattern], int(group_num), int(window), int(block), int(offset), int(n_sink))
+    n_work = _C.intra_llm_bwd_workspace(B, S, H, k.shape[2], *args)
+    if n_work < 0:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
     dq, dk, dv = (torch.empty(t.shape, dtype=t.dtype, device=t.device) for t in (q, k, v))
-    work = torch.empty(B, H, S, dtype=torch.float32, device=q.device)
+    work = torch.empty(n_work, dtype=torch.float32, device=q.device)
     guard, stream = _stream_on(q.device)
     with guard:
         rc = _C.intra_llm_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), dout.data_ptr(),
                               dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), work.data_ptr(), B, S, H, k.shape[2],
                               _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
                               _lib.strides3(dout), _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv),
-                              _lib.strides3(lse), ids[pattern], int(group_num), int(window), int(block), 0, 0,
-                              float(_scale(q, softmax_scale)), stream)
+                              _lib.strides3(lse), *args, float(_scale(q, softmax_scale)), stream)
     if rc != _lib.INTRA_OK:
         raise RuntimeError(f"intra_hip: {_lib.last_error()}")
     return dq, dk, dv
@@ -162,23 +166,24 @@ def intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", group_num=8, 
 
 class _LlmAttnFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, q, k, v, pattern, group_num, window, softmax_scale, block):
-        out, lse = intra_llm_attn(q, k, v, pattern, group_num, window, softmax_scale, return_lse=True, block=block)
+    def forward(ctx, q, k, v, pattern, group_num, window, softmax_scale, block, offset, n_sink):
+        out, lse = intra_llm_attn(q, k, v, pattern, group_num, window, softmax_scale, return_lse=True, block=block,
+                                  offset=offset, n_sink=n_sink)
         ctx.save_for_backward(q, k, v, out, lse)
-        ctx.args = (pattern, group_num, window, softmax_scale, block)
+        ctx.args = (pattern, group_num, window, softmax_scale, block, offset, n_sink)
         return out
 
     @staticmethod
     def backward(ctx, dout):
         q, k, v, out, lse = ctx.saved_tensors
         dq, dk, dv = intra_llm_attn_bwd(q, k, v, out, lse, dout, *ctx.args)
-        return dq, dk, dv, None, None, None, None, None
+        return (dq, dk, dv) + (None,) * 7
 
 
-def intra_llm_attn_func(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None, block=256):
-    """intra_llm_attn as a differentiable function (torch.autograd) for the patterns that
-    intra_llm_attn_bwd covers."""
-    return _LlmAttnFunction.apply(q, k, v, pattern, group_num, window, softmax_scale, block)
+def intra_llm_attn_func(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None, block=256, offset=0,
+                        n_sink=0):
+    """intra_llm_attn as a differentiable function (torch.autograd): forward and backward kernels."""
+    return _LlmAttnFunction.apply(q, k, v, pattern, group_num, window, softmax_scale, block, offset, n_sink)
 
 
 def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None, return_lse=False):

@@ -135,9 +135,51 @@ def test_autograd_function_matches_dense_autograd():
     compare((q.grad, k.grad, v.grad), want, "autograd")
 
 
-def test_unsupported_patterns_raise():
-    q, k, v, dout = make(1, 512, 4, 4)
+@pytest.mark.parametrize("S,kw", [
+    (2000, dict(group_num=2, block=256, offset=1, n_sink=64)),   # the LLaMA setting of the reference's model code
+    (2000, dict(group_num=2, block=256, offset=0, n_sink=64)),
+    (2100, dict(group_num=4, block=256, offset=3, n_sink=0)),
+    (1300, dict(group_num=3, block=512, offset=2, n_sink=100)),
+    (1111, dict(group_num=3, block=64, offset=0, n_sink=40)),
+    (200, dict(group_num=2, block=256, offset=1, n_sink=64)),
+    (4096, dict(group_num=2, block=256, offset=1, n_sink=256)),
+])
+@pytest.mark.parametrize("B,H,Hkv", [(1, 8, 2), (2, 2, 2)])
+def test_block_scatter_offsets_and_sinks_grads(S, kw, B, H, Hkv):
+    run_case("llm/block_scatter", "block_scatter", B, S, H, Hkv, **kw)
+
+
+@pytest.mark.parametrize("S,kw", [
+    (1500, dict(window=575, n_sink=64)), (700, dict(window=1, n_sink=3)), (600, dict(window=100, n_sink=300)),
+    (500, dict(window=5000, n_sink=0)), (3000, dict(window=64, n_sink=0)), (2500, dict(window=300, n_sink=17)),
+])
+@pytest.mark.parametrize("B,H,Hkv", [(1, 8, 2), (2, 3, 3)])
+def test_window_sink_grads(S, kw, B, H, Hkv):
+    run_case("llm/window_sink", "window_sink", B, S, H, Hkv, **kw)
+
+
+def test_model_setting_at_16k():
+    run_case("llm/block_scatter", "block_scatter", 1, 16384, 8, 2, group_num=2, block=256, offset=1, n_sink=64)
+    run_case("llm/window_sink", "window_sink", 1, 16384, 8, 2, window=575, n_sink=64)
+
+
+def test_autograd_function_with_sinks():
+    B, S, H, Hkv = 1, 1024, 4, 2
+    q, k, v, _ = make(B, S, H, Hkv, seed=3)
+    q, k, v = (t.requires_grad_(True) for t in (q, k, v))
+    out = intra_llm_attn_func(q, k, v, "window_sink", window=200, n_sink=16)
+    w = torch.linspace(-1, 1, 128, device=DEV)
+    (out.float() * w).sum().backward()
+    dout = w.expand_as(out).to(torch.bfloat16)
+    mask = oracle.mask_rows("llm/window_sink", S, device=DEV, window=200, n_sink=16)
+    compare((q.grad, k.grad, v.grad), oracle.masked_attention_grads(q, k, v, dout, mask), "autograd with sinks")
+
+
+def test_unsupported_requests_raise():
+    q, k, v, dout = make(1, 512, 8, 4)  # two query heads per kv head: the forward takes 128-token blocks
     with torch.no_grad():
-        out, lse = intra_llm_attn(q, k, v, "window_sink", window=100, n_sink=4, return_lse=True)
+        out, lse = intra_llm_attn(q, k, v, "block_scatter", group_num=2, block=128, offset=1, return_lse=True)
+    with pytest.raises(RuntimeError, match="block % 256"):
+        intra_llm_attn_bwd(q, k, v, out, lse, dout, "block_scatter", group_num=2, block=128, offset=1)
     with pytest.raises(ValueError):
-        intra_llm_attn_bwd(q, k, v, out, lse, dout, "window_sink", window=100)
+        intra_llm_attn_bwd(q, k, v, out, lse, dout, "gather0")

@@ -17,7 +17,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_exports_every_declared_symbol(lib):
     header = open(os.path.join(ROOT, "include", "intra_hip.h")).read()
-    declared = set(re.findall(r"^\s*(?:const\s+char\*|int)\s+(intra_\w+)\s*\(", header, re.M))
+    declared = set(re.findall(r"^\s*(?:const\s+char\*|int|int64_t)\s+(intra_\w+)\s*\(", header, re.M))
     assert declared == set(_lib.SYMBOLS), (declared, set(_lib.SYMBOLS))
     for name in declared:
         assert getattr(lib, name) is not None
@@ -242,8 +242,45 @@ def test_bwd_validates_before_touching_the_gpu(lib):
     assert call(scale=float("nan")) == _lib.INTRA_ERR_INVALID
     assert call(H=6, Hkv=4) == _lib.INTRA_ERR_INVALID
     assert call(pattern=7) == _lib.INTRA_ERR_INVALID
-    # patterns whose dk / dv are not built
-    assert call(pattern=9, window=100) == _lib.INTRA_ERR_UNSUPPORTED
-    assert call(pattern=8, offset=1) == _lib.INTRA_ERR_UNSUPPORTED
-    assert call(pattern=8, n_sink=4) == _lib.INTRA_ERR_UNSUPPORTED
+    assert call(scale=0.0) == _lib.INTRA_ERR_UNSUPPORTED
+    # a stripe offset needs key row blocks inside one block
+    assert call(pattern=8, offset=1, block=128) == _lib.INTRA_ERR_UNSUPPORTED
     assert "backward" in _lib.last_error()
+    assert call(ptrs=(P,) * 9 + (P + 4,)) == _lib.INTRA_ERR_INVALID and "workspace" in _lib.last_error()
+
+
+def test_bwd_workspace_size(lib):
+    assert lib.intra_llm_bwd_workspace(1, 1000, 8, 2, 0, 8, 576, 256, 0, 0) == 8000
+    assert lib.intra_llm_bwd_workspace(2, 1001, 3, 3, 4, 8, 576, 256, 0, 0) == 6008  # rounded up to 4
+    # sinks: ceil(S / 1024) chunks x B x Hkv x n_sink x 128 more
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 24000 + 3 * 2 * 64 * 128
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 256, 1, 0) == 24000
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 128, 1, 0) == -1
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 3, 0, 8, 576, 256, 0, 0) == -1
+
+
+BWD_CASES = [
+    (0, "llm/scatter", 1000, dict(group_num=3)), (0, "llm/scatter", 63, dict(group_num=8)),
+    (1, "llm/gather1", 1024, dict(group_num=8)), (4, "llm/window", 1000, dict(window=192)),
+    (4, "llm/window", 300, dict(window=64)),
+    (8, "llm/block_scatter", 1500, dict(group_num=2, block=256)),
+    (8, "llm/block_scatter", 1111, dict(group_num=3, block=64, n_sink=40)),
+    (8, "llm/block_scatter", 2000, dict(group_num=2, block=256, offset=1, n_sink=64)),
+    (8, "llm/block_scatter", 2100, dict(group_num=4, block=256, offset=3)),
+    (8, "llm/block_scatter", 1300, dict(group_num=3, block=512, offset=2, n_sink=512)),
+    (8, "llm/block_scatter", 200, dict(group_num=2, block=256, offset=1, n_sink=64)),
+    (9, "llm/window_sink", 1500, dict(window=575, n_sink=64)), (9, "llm/window_sink", 700, dict(window=1, n_sink=3)),
+    (9, "llm/window_sink", 600, dict(window=100, n_sink=300)), (9, "llm/window_sink", 500, dict(window=5000, n_sink=0)),
+]
+
+
+@pytest.mark.parametrize("pattern,kind,S,kw", BWD_CASES)
+def test_backward_key_row_maps_equal_mask(lib, pattern, kind, S, kw):
+    """Every (query, key) pair of the mask is multiplied exactly once by the dk / dv launches
+    (inverse index maps, unsaved sink rows, sink pass)."""
+    count = np.zeros((S, S), dtype=np.uint8)
+    rc = lib.intra_model_mask_llm_bwd(pattern, S, kw.get("group_num", 2), kw.get("window", 575), kw.get("block", 256),
+                                      kw.get("offset", 0), kw.get("n_sink", 0), count.ctypes.data)
+    assert rc == 0, _lib.last_error()
+    want = oracle.mask_rows(kind, S, **kw).numpy().astype(np.uint8)
+    assert np.array_equal(count, want), np.argwhere(count != want)[:5]
