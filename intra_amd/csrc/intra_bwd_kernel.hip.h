@@ -1,6 +1,7 @@
-// Backward kernels of the sparse attention for gfx950 (MI355X): dQ, dK and dV for the patterns
-// whose sets number queries and keys alike and whose rows meet one contiguous range of columns
-// (LLM Scatter, Gather 1, 64-aligned window, block Scatter without offset and sinks).
+// Backward kernels of the sparse attention for gfx950 (MI355X): dQ, dK and dV for the causal LLM
+// patterns (Scatter, Gather 1, 64-aligned window, block Scatter with stripe offsets and sinks,
+// per-token window with sinks).  Which rows meet which columns comes from the row maps of
+// intra_bwd_maps.h.
 //
 // The reference has no backward kernels (its README names them as missing; training there runs
 // through masked SDPA / FlexAttention, experiments/llm/llama_intra.py:26).  The math is the usual
@@ -14,9 +15,7 @@
 // columns a wavefront forms the scores S^T = C1 R1^T and dP^T = C2 R2^T, turns them into the
 // weights (P or dS), packed to bf16 straight from the accumulators, and adds X^T W^T to its
 // accumulators, X being the K, Q or dO tile read with transposing LDS reads - the data flow of
-// the forward kernel without the online softmax.  Which columns a row meets follows from the same
-// index maps; for dK / dV the query range of a key is found by bisection on the maps' monotone
-// bounds, so no pattern needs inverse formulas.
+// the forward kernel without the online softmax.
 #pragma once
 #include "intra_bwd_maps.h"
 #include "intra_kernel.hip.h"
