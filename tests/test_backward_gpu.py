@@ -183,3 +183,74 @@ def test_unsupported_requests_raise():
         intra_llm_attn_bwd(q, k, v, out, lse, dout, "block_scatter", group_num=2, block=128, offset=1)
     with pytest.raises(ValueError):
         intra_llm_attn_bwd(q, k, v, out, lse, dout, "gather0")
+
+
+def test_c_abi_with_packed_gradient_buffer_and_strided_lse():
+    """The C ABI directly: dq, dk, dv written into slices of one packed (B, S, H + 2 Hkv, 128)
+    gradient buffer, lse passed with (batch, head, token) strides of a (B, S, H) tensor, and a
+    workspace of exactly the size the library asks for."""
+    from intra_amd import _lib
+    lib = _lib.load()
+    B, S, H, Hkv = 2, 1000, 8, 2
+    q, k, v, dout = make(B, S, H, Hkv, seed=11)
+    kw = dict(window=200, n_sink=24)
+    with torch.no_grad():
+        out, lse = intra_llm_attn(q, k, v, "window_sink", return_lse=True, **kw)
+    lse_t = lse.transpose(1, 2).contiguous()  # (B, S, H) storage
+    lse_st = _lib._i64x3(lse_t.stride(0), lse_t.stride(2), lse_t.stride(1))
+    grads = torch.full((B, S, H + 2 * Hkv, 128), float("nan"), dtype=torch.bfloat16, device=DEV)
+    dq, dk, dv = grads[:, :, :H], grads[:, :, H:H + Hkv], grads[:, :, H + Hkv:]
+    n = lib.intra_llm_bwd_workspace(B, S, H, Hkv, 9, 2, 200, 256, 0, 24)
+    assert n == B * H * S + 1 * B * Hkv * 24 * 128
+    work = torch.full((n + 64,), float("nan"), dtype=torch.float32, device=DEV)  # NaN: contents must not matter
+    rc = lib.intra_llm_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse_t.data_ptr(), dout.data_ptr(),
+                           dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), work.data_ptr(), B, S, H, Hkv,
+                           _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out), _lib.strides3(dout),
+                           _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv), lse_st, 9, 2, 200, 256, 0, 24,
+                           128 ** -0.5, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(work[n:]).all()), "wrote past the workspace"
+    mask = oracle.mask_rows("llm/window_sink", S, device=DEV, **kw)
+    compare((dq, dk, dv), oracle.masked_attention_grads(q, k, v, dout, mask), "packed gradients")
+
+
+def test_results_do_not_change_between_calls():
+    """No atomics anywhere (the sink rows are summed in a fixed order): bit-identical reruns."""
+    q, k, v, dout = make(1, 3000, 8, 2, seed=5)
+    kw = dict(group_num=2, block=256, offset=1, n_sink=64)
+    a = kernel_grads(q, k, v, dout, "block_scatter", **kw)
+    b = kernel_grads(q, k, v, dout, "block_scatter", **kw)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+def test_backward_can_be_captured_in_a_graph_and_replayed():
+    """Forward + backward allocate only through torch and record no memset, so they can go into a
+    HIP graph; every replay, with fresh inputs copied into the captured tensors and eager work in
+    between, must equal the eager result."""
+    B, S, H, Hkv = 1, 1024, 8, 2
+    kw = dict(window=300, n_sink=32)
+    sq, sk, sv, sd = make(B, S, H, Hkv, seed=20)
+    stream = torch.cuda.Stream()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream), torch.no_grad():
+        for _ in range(2):  # warm-up outside the capture
+            o, l = intra_llm_attn(sq, sk, sv, "window_sink", return_lse=True, **kw)
+            intra_llm_attn_bwd(sq, sk, sv, o, l, sd, "window_sink", **kw)
+    torch.cuda.current_stream().wait_stream(stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), torch.no_grad():
+        o, l = intra_llm_attn(sq, sk, sv, "window_sink", return_lse=True, **kw)
+        gq, gk, gv = intra_llm_attn_bwd(sq, sk, sv, o, l, sd, "window_sink", **kw)
+    for seed in (21, 22, 23):
+        nq, nk, nv, nd = make(B, S, H, Hkv, seed=seed)
+        for dst, src in ((sq, nq), (sk, nk), (sv, nv), (sd, nd)):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = kernel_grads(nq, nk, nv, nd, "window_sink", **kw)
+        torch.cuda.synchronize()
+        for x, y in zip((gq, gk, gv), eager):
+            assert torch.equal(x, y), f"replay with seed {seed} differs from the eager call"
