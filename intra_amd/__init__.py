@@ -1,4 +1,4 @@
-"""MI355X-native INTRA sparse attention (forward).  Mirrors intra_attn/__init__.py:1-9 of the
+"""MI355X-native INTRA sparse attention (forward kernels of the reference, plus a backward pass).  Mirrors intra_attn/__init__.py:1-9 of the
 reference: if the native library is missing, both entry points raise ImportError when called."""
 try:
     from .interface import intra_image_attn, intra_llm_attn, intra_llm_attn_bwd, intra_llm_attn_func
