@@ -78,3 +78,48 @@ def test_image_patterns(lib, w8, t8, hp, gather0):
     kind = "image/gather0" if gather0 else "image/scatter"
     want = oracle.mask_rows(kind, S, width=W, text_len=T)
     assert torch.equal(torch.from_numpy(count), want.to(torch.uint8))
+
+
+# ---------------------------------------------------------------------------- backward (dk / dv launches)
+def _walk_bwd(lib, pattern, S, group_num=8, window=576, block=256, offset=0, n_sink=0):
+    count = np.zeros((S, S), dtype=np.uint8)
+    rc = lib.intra_model_mask_llm_bwd(pattern, S, group_num, window, block, offset, n_sink, count.ctypes.data)
+    return rc, torch.from_numpy(count)
+
+
+@settings(**COMMON)
+@given(S=st.integers(1, 1400), G=st.integers(1, 40), gather=st.booleans())
+def test_backward_scatter_and_gather1(lib, S, G, gather):
+    rc, count = _walk_bwd(lib, 1 if gather else 0, S, group_num=G)
+    assert rc == 0, _lib.last_error()
+    kind = "llm/gather1" if gather else "llm/scatter"
+    assert torch.equal(count, oracle.mask_rows(kind, S, group_num=G).to(torch.uint8))
+
+
+@settings(**COMMON)
+@given(S=st.integers(1, 1400), W=st.integers(64, 3000))
+def test_backward_aligned_window(lib, S, W):
+    rc, count = _walk_bwd(lib, 4, S, window=W)
+    assert rc == 0, _lib.last_error()
+    assert torch.equal(count, oracle.mask_rows("llm/window", S, window=W).to(torch.uint8))
+
+
+@settings(**COMMON)
+@given(S=st.integers(1, 2600), W=st.integers(1, 2000), ns=st.integers(0, 1500))
+def test_backward_window_with_sinks(lib, S, W, ns):
+    rc, count = _walk_bwd(lib, 9, S, window=W, n_sink=ns)
+    assert rc == 0, _lib.last_error()
+    assert torch.equal(count, oracle.mask_rows("llm/window_sink", S, window=W, n_sink=ns).to(torch.uint8))
+
+
+@settings(**COMMON)
+@given(S=st.integers(1, 2600), G=st.integers(1, 6), blk64=st.integers(1, 8), off=st.integers(0, 5), ns_frac=st.floats(0, 1))
+def test_backward_block_scatter(lib, S, G, blk64, off, ns_frac):
+    blk, off = 64 * blk64, off % G
+    if off != 0:
+        blk = 256 * ((blk64 + 1) // 2)  # a stripe offset needs 256-key row blocks inside one block
+    ns = int(ns_frac * blk)
+    rc, count = _walk_bwd(lib, 8, S, group_num=G, block=blk, offset=off, n_sink=ns)
+    assert rc == 0, _lib.last_error()
+    want = oracle.mask_rows("llm/block_scatter", S, group_num=G, block=blk, offset=off, n_sink=ns)
+    assert torch.equal(count, want.to(torch.uint8))
