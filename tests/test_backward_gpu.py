@@ -6,6 +6,7 @@ differentiates in training is the dense-mask attention the oracle restates
 Tolerance, on bf16 results, per tensor with m = max|want|:
   every element  |got - want| <= m / 64 + |want| / 64
   whole tensor   ||got - want||_2 <= ||want||_2 / 128
+(plus 1e-4 per element in both, for gradients that are exactly zero)
 The kernels round the softmax weights and their derivatives to bf16 before the second product
 (2^-9 relative each), use the forward pass's log-sum-exp (within 2^-8 of exact), form
 D = dout . out from the bf16 output, and round the results to bf16 (2^-9).  The terms that add up
@@ -20,6 +21,7 @@ from intra_amd import intra_llm_attn, intra_llm_attn_bwd, intra_llm_attn_func
 
 pytestmark = pytest.mark.gpu
 RTOL, NORM_RTOL = 1.0 / 64, 1.0 / 128
+ABS_FLOOR = 1e-4  # gradients that vanish exactly (one-key rows) come out as fp32 rounding noise of dP - D
 DEV = "cuda"
 
 
@@ -42,10 +44,10 @@ def compare(got, want, what):
         w = w.float()
         diff = (g.float() - w).abs()
         m = w.abs().max().item()
-        ok = diff <= RTOL * m + RTOL * w.abs()
+        ok = diff <= RTOL * m + RTOL * w.abs() + ABS_FLOOR
         assert bool(ok.all()), f"{what} {name}: max|err|={diff.max().item():.3e}, max|want|={m:.3e}"
-        rel = (diff.norm() / w.norm()).item()
-        assert rel <= NORM_RTOL, f"{what} {name}: relative l2 error {rel:.3e}"
+        bound = NORM_RTOL * w.norm().item() + ABS_FLOOR * w.numel() ** 0.5
+        assert diff.norm().item() <= bound, f"{what} {name}: l2 error {diff.norm().item():.3e} > {bound:.3e}"
 
 
 def run_case(kind, pattern, B, S, H, Hkv, seed=0, scale=None, mask_kw=None, **kw):
@@ -254,3 +256,37 @@ def test_backward_can_be_captured_in_a_graph_and_replayed():
         torch.cuda.synchronize()
         for x, y in zip((gq, gk, gv), eager):
             assert torch.equal(x, y), f"replay with seed {seed} differs from the eager call"
+
+
+def _random_cases(n, seed):
+    import random
+    rnd = random.Random(seed)
+    heads = [(4, 4), (4, 2), (8, 2), (4, 1), (16, 4), (3, 3), (6, 3)]
+    cases = []
+    for _ in range(n):
+        H, Hkv = rnd.choice(heads)
+        B = rnd.choice([1, 1, 2])
+        S = rnd.choice([rnd.randint(1, 300), rnd.randint(300, 2500), 64 * rnd.randint(1, 36)])
+        kind = rnd.choice(["scatter", "gather1", "window", "block_scatter", "window_sink"])
+        if kind == "scatter":
+            kw = dict(group_num=rnd.choice([1, 2, 3, 5, 8, 13]))
+        elif kind == "gather1":
+            S = 64 * max(1, S // 64)
+            kw = dict(group_num=8)
+        elif kind == "window":
+            kw = dict(window=rnd.choice([64, 65, 128, 576, 1000, 4000]))
+        elif kind == "block_scatter":
+            G = rnd.choice([1, 2, 3, 4])
+            off = rnd.randrange(G)
+            blk = 256 * rnd.choice([1, 1, 2]) if (off or (H // Hkv) % 4) else 64 * rnd.choice([1, 2, 4, 8])
+            kw = dict(group_num=G, block=blk, offset=off, n_sink=rnd.choice([0, 1, 64, blk]))
+        else:
+            kw = dict(window=rnd.choice([1, 2, 63, 64, 575, 2000]), n_sink=rnd.choice([0, 1, 64, 100, 700]))
+        cases.append((kind, B, S, H, Hkv, kw, rnd.choice([None, None, 0.05, -0.11])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(40, seed=77), ids=lambda c: f"{c[0]}-S{c[2]}-H{c[3]}/{c[4]}")
+def test_random_shapes(case):
+    kind, B, S, H, Hkv, kw, scale = case
+    run_case(f"llm/{kind}", kind, B, S, H, Hkv, seed=S + H, scale=scale, **kw)
