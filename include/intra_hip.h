@@ -127,9 +127,10 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
                   const int64_t dk_strides[3], const int64_t dv_strides[3],
                   const int64_t lse_strides[3], int pattern, int group_num, int window, int block,
                   int offset, int n_sink, float softmax_scale, void* hip_stream);
-/* Floats of workspace that intra_llm_bwd needs for such a call (B*H*S rounded up to 4, plus
- * ceil(S/1024) * B * Hkv * min(n_sink, S) * 128 with sinks); -1 if the request is invalid or
- * unsupported (intra_last_error() says why).  No counterpart in the reference. */
+/* Floats of workspace that intra_llm_bwd needs for such a call (B*H*S rounded up to 4, plus with
+ * sinks chunks * B * Hkv * min(n_sink, S) * 128, the queries being cut into chunks of 128 to
+ * 1024 so that the sink pass fills the GPU); -1 if the request is invalid or unsupported
+ * (intra_last_error() says why).  No counterpart in the reference. */
 int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int group_num,
                                 int window, int block, int offset, int n_sink);
 

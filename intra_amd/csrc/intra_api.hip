@@ -43,6 +43,8 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   r->H = H;
   r->Hkv = Hkv;
   r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1, 64, 0, 0};  // derived fields: geom_finish() in shape_for()
+  // sink pass of the backward: about 512 workgroups, 128..1024 queries each
+  r->geom.sink_chunk = (int)std::min<int64_t>(1024, std::max<int64_t>(128, 64 * (((int64_t)S * B * Hkv + 512 * 64 - 1) / (512 * 64))));
   if (domain == 0) {
     if (!extended && (pattern == INTRA_LLM_BLOCK_SCATTER || pattern == INTRA_LLM_WINDOW_SINK))
       return fail(INTRA_ERR_INVALID, "unknown LLM pattern id %d (0 scatter, 1 gather1, 4 window)", pattern);
@@ -464,7 +466,7 @@ int64_t bwd_workspace_floats(const Request& r) {
   int64_t n = bwd_dsum_floats(r.B, r.S, r.H);
   const int ns = std::min(r.geom.ns, r.S);
   if ((r.kind == KIND_LLM_BLOCK_SCATTER || r.kind == KIND_LLM_WINDOW_SINK) && ns > 0)
-    n += (int64_t)((r.S + intra::SINK_CHUNK - 1) / intra::SINK_CHUNK) * r.B * r.Hkv * ns * 128;
+    n += (int64_t)((r.S + r.geom.sink_chunk - 1) / r.geom.sink_chunk) * r.B * r.Hkv * ns * 128;
   return n;
 }
 

@@ -21,8 +21,6 @@
 
 namespace intra {
 
-constexpr int SINK_CHUNK = 1024;  // queries per workgroup of the sink pass
-
 template <class MAP>
 struct QueryRows {
   MAP m;
@@ -47,10 +45,9 @@ struct QueryRows {
 template <class MAP>
 struct KeyRowsOf {
   MAP m;
-  int skip;
   static IM_HD int num_sets(const IntraGeom& ge) { return MAP::num_sets(ge); }
   static IM_HD int max_rows(const IntraGeom& ge) { return MAP::max_nq(ge); }
-  IM_HD KeyRowsOf(const IntraGeom& ge, int set, int) : m(ge, set, 0), skip(0) {}
+  IM_HD KeyRowsOf(const IntraGeom& ge, int set, int) : m(ge, set, 0) {}
   IM_HD int n_rows() const { return m.nk(); }
   IM_HD int n_cols() const { return m.nq(); }
   IM_HD int kpre() const { return 0; }
@@ -162,16 +159,17 @@ struct KeyRowsWindowSink {
 };
 
 // The sink keys (positions below n_sink) against every later query of the sequence; set = chunk
-// of SINK_CHUNK queries.  The results are partial sums over the chunk.
+// of ge.sink_chunk queries (chosen by the host so that the pass fills the GPU).  The results are
+// partial sums over the chunk.
 struct KeyRowsSinks {
   int S, ns, c0, c1;
-  static IM_HD int num_sets(const IntraGeom& ge) { return (ge.S + SINK_CHUNK - 1) / SINK_CHUNK; }
+  static IM_HD int num_sets(const IntraGeom& ge) { return (ge.S + ge.sink_chunk - 1) / ge.sink_chunk; }
   static IM_HD int max_rows(const IntraGeom& ge) { return im_min(ge.ns, ge.S); }
   IM_HD KeyRowsSinks(const IntraGeom& ge, int set, int) {
     S = ge.S;
     ns = im_min(ge.ns, ge.S);
-    c0 = set * SINK_CHUNK;
-    c1 = im_min(c0 + SINK_CHUNK, S);
+    c0 = set * ge.sink_chunk;
+    c1 = im_min(c0 + ge.sink_chunk, S);
   }
   IM_HD int n_rows() const { return ns; }
   IM_HD int n_cols() const { return S; }

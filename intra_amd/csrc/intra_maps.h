@@ -79,6 +79,7 @@ struct IntraGeom {
   int blk;       // LLM block scatter: tokens per block
   int off;       // LLM block scatter: stripe offset, 0 <= off < G
   int ns;        // LLM block scatter / window with sinks: leading tokens every query sees
+  int sink_chunk;  // backward: queries per workgroup of the sink pass (a multiple of 64)
   // derived by geom_finish()
   FastDiv dG;        // / G
   FastDiv dWq;       // / (width / 4)

@@ -252,8 +252,10 @@ def test_bwd_validates_before_touching_the_gpu(lib):
 def test_bwd_workspace_size(lib):
     assert lib.intra_llm_bwd_workspace(1, 1000, 8, 2, 0, 8, 576, 256, 0, 0) == 8000
     assert lib.intra_llm_bwd_workspace(2, 1001, 3, 3, 4, 8, 576, 256, 0, 0) == 6008  # rounded up to 4
-    # sinks: ceil(S / 1024) chunks x B x Hkv x n_sink x 128 more
-    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 24000 + 3 * 2 * 64 * 128
+    # sinks: chunks x B x Hkv x n_sink x 128 more; chunks of 128 queries here (64 * ceil(S*B*Hkv / 32768), at least 128)
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 24000 + 24 * 2 * 64 * 128
+    # ... of 1024 queries for long sequences
+    assert lib.intra_llm_bwd_workspace(1, 65536, 32, 8, 9, 2, 575, 256, 0, 64) == 65536 * 32 + 64 * 8 * 64 * 128
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 256, 1, 0) == 24000
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 128, 1, 0) == -1
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 3, 0, 8, 576, 256, 0, 0) == -1
