@@ -131,6 +131,28 @@ def main():
             "sample": f"{n_rows} evenly spaced query rows x {H} heads of the same S={S} problem, dense-mask fp32 "
                       f"oracle, {dt:.2f} s; dense work {4.0 * 128 * n_rows * S * H / dt / 1e12:.4f} TFLOP/s",
         }
+        # the reference's CPU-runnable case beside it, whole problem on both sides: Scatter G=8,
+        # S=1024, 4 query / 1 kv heads (median of 5 runs after a warm-up)
+        qs, ks, vs = (t[:, :1024, :n].contiguous() for t, n in ((q_cpu, 4), (k_cpu, 1), (v_cpu, 1)))
+        mask_s = oracle.llm_scatter_mask(1024, G)
+        cpu_ms = []
+        for _ in range(6):
+            t0 = time.perf_counter()
+            oracle.masked_attention(qs, ks, vs, mask_s)
+            cpu_ms.append((time.perf_counter() - t0) * 1e3)
+        qg, kg, vg = qs.to(dev), ks.to(dev), vs.to(dev)
+        gpu_ms = []
+        with torch.no_grad():
+            for i in range(8):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                intra_llm_attn(qg, kg, vg, "scatter", group_num=G)
+                b.record()
+                torch.cuda.synchronize()
+                gpu_ms.append(a.elapsed_time(b))
+        res["cpu_baseline"]["small_case"] = {
+            "workload": f"LLM causal Scatter G={G}, B=1, S=1024, 4 query / 1 kv heads",
+            "cpu_ms": round(sorted(cpu_ms[1:])[2], 3), "gpu_ms": round(sorted(gpu_ms[3:])[2], 4)}
     print(json.dumps(res), flush=True)
 
 
