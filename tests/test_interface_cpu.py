@@ -75,3 +75,30 @@ def test_product_never_imports_the_oracle():
             if name.endswith(".py"):
                 text = open(os.path.join(root, pkg, name)).read()
                 assert "import oracle" not in text and "from oracle" not in text, f"{pkg}/{name}"
+
+
+def test_llama_caller_module_configuration_on_cpu():
+    """install_intra_llama / set_dense_debug are host logic: schedule, block and stripe offsets per layer."""
+    import types
+
+    from intra_amd.llama_attention import install_intra_llama, set_dense_debug
+    model = types.SimpleNamespace(model=types.SimpleNamespace(
+        layers=[types.SimpleNamespace(self_attn=types.SimpleNamespace()) for _ in range(32)]))
+    counts = install_intra_llama(model, num_groups=2, window=575, n_sink=64, scatter_blocks=(256,),
+                                 layer_pattern="SWWWWWWW", scatter_stripe=True, scatter_n_offsets=2)
+    assert counts == (4, 28, 0)
+    cfgs = [l.self_attn._intra for l in model.model.layers]
+    assert [c["layer_idx"] for c in cfgs if c["kind"] == "S"] == [0, 8, 16, 24]
+    assert [c["scatter_offset"] for c in cfgs if c["kind"] == "S"] == [0, 1, 0, 1]
+    assert all(c["scatter_block"] == 256 for c in cfgs if c["kind"] == "S")
+    assert all(c["window"] == 575 and c["n_sink"] == 64 for c in cfgs)
+    set_dense_debug(model, True)
+    assert all(c["dense_debug"] for c in cfgs)
+    # without stripes every Scatter layer has offset 0; blocks cycle over the Scatter layers
+    counts = install_intra_llama(model, num_groups=8, scatter_blocks=(64, 128), layer_pattern="sd?w")
+    assert counts == (11, 10, 11)
+    s_cfgs = [l.self_attn._intra for l in model.model.layers if l.self_attn._intra["kind"] == "S"]
+    assert [c["scatter_block"] for c in s_cfgs[:4]] == [64, 128, 64, 128]
+    assert all(c["scatter_offset"] == 0 for c in s_cfgs)
+    with pytest.raises(ValueError):
+        install_intra_llama(model, num_groups=2, scatter_blocks=(128,), layer_pattern="S", scatter_stripe=True)

@@ -1,0 +1,129 @@
+"""The call pattern of the reference's LLaMA / Qwen integration (experiments/llm/llama_intra.py:
+177-221, 232-270) without model weights: a small decoder stack with random projections whose
+attention goes through intra_amd.llama_attention.intra_attention_forward, forward and backward,
+against the same stack on masked SDPA with the oracle's masks (what the reference trains with,
+llama_intra.py:26).  Inputs reach the kernels as transposed (B, H, S, D) views of the projection
+outputs, with GQA, an explicit scaling and the "g2s4" layer schedule: Scatter layers with stripe
+offsets 0 / 1 and window layers, all with sinks.
+
+Tolerance: both stacks compute in bf16; outputs and every gradient agree to a relative l2 error of
+3e-2 (observed about 1e-2, the level of two bf16 implementations of the same layer stack)."""
+import types
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+from intra_amd.llama_attention import install_intra_llama, intra_attention_forward, set_dense_debug
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+HQ, HKV, D = 4, 2, 128
+HIDDEN = HQ * D
+
+
+def make_model(n_layers, seed):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    w = lambda o, i: (torch.randn(o, i, generator=g) * i ** -0.5).to(torch.bfloat16).to(DEV).requires_grad_(True)
+    layers = []
+    for _ in range(n_layers):
+        attn = types.SimpleNamespace(scaling=D ** -0.5, wq=w(HQ * D, HIDDEN), wk=w(HKV * D, HIDDEN),
+                                     wv=w(HKV * D, HIDDEN), wo=w(HIDDEN, HQ * D))
+        layers.append(types.SimpleNamespace(self_attn=attn))
+    return types.SimpleNamespace(layers=layers)
+
+
+def masked_sdpa_forward(module, query, key, value, attention_mask=None, scaling=None, dropout=0.0, **kwargs):
+    """The same interface on dense-mask SDPA, masks from the oracle."""
+    cfg, S = module._intra, query.shape[2]
+    if cfg["kind"] == "S":
+        mask = oracle.mask_rows("llm/block_scatter", S, device=DEV, group_num=cfg["num_groups"], block=cfg["scatter_block"],
+                                offset=cfg["scatter_offset"], n_sink=cfg["n_sink"])
+    elif cfg["kind"] == "W":
+        mask = oracle.mask_rows("llm/window_sink", S, device=DEV, window=cfg["window"], n_sink=cfg["n_sink"])
+    else:
+        mask = torch.ones(S, S, dtype=torch.bool, device=DEV).tril()
+    out = F.scaled_dot_product_attention(query, key, value, attn_mask=mask, scale=scaling, enable_gqa=True)
+    return out.transpose(1, 2).contiguous(), None
+
+
+def run_stack(model, x, attention):
+    B, S, _ = x.shape
+    for layer in model.layers:
+        a = layer.self_attn
+        h = F.rms_norm(x, (HIDDEN,))
+        q = (h @ a.wq.T).view(B, S, HQ, D).transpose(1, 2)   # (B, H, S, D) views, as transformers passes them
+        k = (h @ a.wk.T).view(B, S, HKV, D).transpose(1, 2)
+        v = (h @ a.wv.T).view(B, S, HKV, D).transpose(1, 2)
+        out, _ = attention(a, q, k, v, attention_mask=None, scaling=a.scaling, dropout=0.0)
+        assert out.shape == (B, S, HQ, D) and out.is_contiguous()
+        x = x + out.reshape(B, S, HIDDEN) @ a.wo.T
+    return x
+
+
+def params(model):
+    return [w for layer in model.layers for w in (layer.self_attn.wq, layer.self_attn.wk, layer.self_attn.wv, layer.self_attn.wo)]
+
+
+def rel(a, b):
+    return ((a.float() - b.float()).norm() / b.float().norm()).item()
+
+
+@pytest.mark.parametrize("S", [1024, 1300])
+def test_g2s4_stack_forward_and_backward(S):
+    B = 2
+    model = make_model(8, seed=1)
+    counts = install_intra_llama(model, num_groups=2, window=200, n_sink=64, scatter_blocks=(256,),
+                                 layer_pattern="SWWW", scatter_stripe=True, scatter_n_offsets=2)
+    assert counts == (2, 6, 0)
+    assert [l.self_attn._intra["scatter_offset"] for l in model.layers if l.self_attn._intra["kind"] == "S"] == [0, 1]
+    g = torch.Generator(device="cpu").manual_seed(2)
+    x0 = torch.randn(B, S, HIDDEN, generator=g).to(torch.bfloat16).to(DEV)
+    results = []
+    for attention in (intra_attention_forward, masked_sdpa_forward):
+        x = x0.clone().requires_grad_(True)
+        for w in params(model):
+            w.grad = None
+        y = run_stack(model, x, attention)
+        y.float().square().mean().backward()
+        results.append((y.detach(), x.grad, [w.grad.clone() for w in params(model)]))
+    (y1, gx1, gw1), (y2, gx2, gw2) = results
+    assert rel(y1, y2) <= 3e-2, rel(y1, y2)
+    assert rel(gx1, gx2) <= 3e-2, rel(gx1, gx2)
+    for i, (a, b) in enumerate(zip(gw1, gw2)):
+        assert torch.isfinite(a).all() and rel(a, b) <= 3e-2, (i, rel(a, b))
+
+
+def test_inference_decode_and_dense_branches():
+    model = make_model(2, seed=3)
+    install_intra_llama(model, num_groups=2, window=128, n_sink=16, scatter_blocks=(64,), layer_pattern="SD")
+    attn_s, attn_d = model.layers[0].self_attn, model.layers[1].self_attn
+    g = torch.Generator(device="cpu").manual_seed(4)
+    mk = lambda h, s: torch.randn(1, h, s, D, generator=g).to(torch.bfloat16).to(DEV)
+    q, k, v = mk(HQ, 700), mk(HKV, 700), mk(HKV, 700)
+    with torch.no_grad():
+        out, _ = intra_attention_forward(attn_s, q, k, v, scaling=0.07)          # prefill, Scatter layer
+        ref, _ = masked_sdpa_forward(attn_s, q, k, v, scaling=0.07)
+        assert (out.float() - ref.float()).abs().max().item() <= 1.6e-2
+        out, _ = intra_attention_forward(attn_d, q, k, v)                        # dense layer
+        ref = F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=D ** -0.5, enable_gqa=True).transpose(1, 2)
+        assert torch.equal(out, ref.contiguous())
+        out, _ = intra_attention_forward(attn_s, q[:, :, -1:], k, v)             # decode: one query, whole cache
+        ref = F.scaled_dot_product_attention(q[:, :, -1:], k, v, scale=D ** -0.5, enable_gqa=True).transpose(1, 2)
+        assert out.shape == (1, 1, HQ, D) and torch.equal(out, ref.contiguous())
+        set_dense_debug(model, True)                                             # teacher toggle
+        out, _ = intra_attention_forward(attn_s, q, k, v)
+        ref = F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=D ** -0.5, enable_gqa=True).transpose(1, 2)
+        assert torch.equal(out, ref.contiguous())
+
+
+def test_configuration_errors():
+    model = make_model(2, seed=5)
+    with pytest.raises(ValueError, match="256"):
+        install_intra_llama(model, num_groups=2, scatter_blocks=(128,), layer_pattern="S", scatter_stripe=True)
+    install_intra_llama(model, num_groups=2, scatter_blocks=(100,), layer_pattern="S")
+    q = torch.zeros(1, HQ, 256, D, dtype=torch.bfloat16, device=DEV)
+    k = torch.zeros(1, HKV, 256, D, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="multiple of 64"):
+        intra_attention_forward(model.layers[0].self_attn, q, k, k)
