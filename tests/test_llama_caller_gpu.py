@@ -127,3 +127,40 @@ def test_configuration_errors():
     k = torch.zeros(1, HKV, 256, D, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError, match="multiple of 64"):
         intra_attention_forward(model.layers[0].self_attn, q, k, k)
+
+
+def test_transformers_llama_model_trains_through_the_kernels():
+    """A randomly initialised transformers LLaMA (tiny: 4 layers, 4 query / 2 kv heads of dim 128,
+    rotary embeddings, RMSNorm, MLP - the real modelling code) with attn_implementation="intra":
+    logits and parameter gradients against the same weights with the masked-SDPA function."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import AttentionInterface, LlamaConfig, LlamaForCausalLM
+
+    from intra_amd import llama_attention
+    llama_attention.register("intra")
+    AttentionInterface.register("intra_masked_sdpa", masked_sdpa_forward)
+    cfg = LlamaConfig(hidden_size=HIDDEN, num_attention_heads=HQ, num_key_value_heads=HKV, head_dim=D, num_hidden_layers=4,
+                      intermediate_size=1024, vocab_size=512, max_position_embeddings=4096)
+    cfg._attn_implementation = "intra"
+    torch.manual_seed(0)
+    model = LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
+    counts = llama_attention.install_intra_llama(model, num_groups=2, window=300, n_sink=64, scatter_blocks=(256,),
+                                                 layer_pattern="SW", scatter_stripe=True, scatter_n_offsets=2)
+    assert counts == (2, 2, 0)
+    ids = torch.randint(0, 512, (2, 1536), generator=torch.Generator().manual_seed(1)).to(DEV)
+    results = []
+    for impl in ("intra", "intra_masked_sdpa"):
+        model.config._attn_implementation = impl
+        for layer in model.model.layers:
+            layer.self_attn.config._attn_implementation = impl
+        model.zero_grad(set_to_none=True)
+        out = model(input_ids=ids, labels=ids, use_cache=False)
+        out.loss.backward()
+        results.append((out.logits.detach().float(), out.loss.item(),
+                        {n: p.grad.detach().float().clone() for n, p in model.named_parameters()}))
+    (l1, loss1, g1), (l2, loss2, g2) = results
+    assert not torch.equal(l1, l2), "both runs took the same attention function"
+    assert abs(loss1 - loss2) <= 2e-2 * abs(loss2), (loss1, loss2)
+    assert rel(l1, l2) <= 3e-2, rel(l1, l2)
+    worst = max((rel(g1[n], g2[n]), n) for n in g1)
+    assert worst[0] <= 5e-2, worst
