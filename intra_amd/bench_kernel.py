@@ -148,6 +148,20 @@ def bench_llm(args):
                     else:
                         intra_llm_attn(ql, kl, vl, "window_sink", window=575, n_sink=64)
             r["g2s4_model_32layer_run"] = round(median_ms(model_stack, 2, max(3, args.iters // 10)), 3)
+            if args.backward:
+                # the same 32 layers forward (with log-sum-exp) and backward: the attention part of a training step
+                douts = [qkv(B, S, H, Hkv, seed=10 + i)[0] for i in range(2)]
+
+                def model_train_stack():
+                    for i in range(32):
+                        ql, kl, vl = layers[i % 4]
+                        if i % 8 == 0:
+                            name, kw = "block_scatter", dict(group_num=2, block=256, offset=(i // 8) % 2, n_sink=64)
+                        else:
+                            name, kw = "window_sink", dict(window=575, n_sink=64)
+                        out, lse = intra_llm_attn(ql, kl, vl, name, return_lse=True, **kw)
+                        intra_llm_attn_bwd(ql, kl, vl, out, lse, douts[i % 2], name, **kw)
+                r["g2s4_model_32layer_fwd_bwd_run"] = round(median_ms(model_train_stack, 1, max(3, args.iters // 10)), 3)
         rows.append(r)
         print(json.dumps(r), flush=True)
     return rows
