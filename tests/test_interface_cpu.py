@@ -102,3 +102,21 @@ def test_llama_caller_module_configuration_on_cpu():
     assert all(c["scatter_offset"] == 0 for c in s_cfgs)
     with pytest.raises(ValueError):
         install_intra_llama(model, num_groups=2, scatter_blocks=(128,), layer_pattern="S", scatter_stripe=True)
+
+
+def test_extension_stand_in_has_the_reference_signatures():
+    """intra_attn_cuda.fwd / fwd_llm take the 16 positional arguments of mha_fwd / mha_fwd_llm
+    (csrc/flash_attn/flash_api.cpp:356-371, 557-574) under the names the pybind module exports
+    (flash_api.cpp:1766-1770)."""
+    import inspect
+
+    import intra_attn_cuda
+    llm = list(inspect.signature(intra_attn_cuda.fwd_llm).parameters)
+    img = list(inspect.signature(intra_attn_cuda.fwd).parameters)
+    assert len(llm) == len(img) == 16
+    assert llm[:3] == img[:3] == ["q", "k", "v"]
+    assert llm[-3:] == ["mask", "group_num", "window"] and img[-3:] == ["mask", "width", "length"]
+    assert llm[5:7] == ["p_dropout", "softmax_scale"]
+    cpu = torch.zeros(1, 64, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        intra_attn_cuda.fwd_llm(cpu, cpu, cpu, None, None, 0.0, 0.1, True, -1, -1, 0.0, False, None, 0, 8, 576)
