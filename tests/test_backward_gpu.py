@@ -290,3 +290,10 @@ def _random_cases(n, seed):
 def test_random_shapes(case):
     kind, B, S, H, Hkv, kw, scale = case
     run_case(f"llm/{kind}", kind, B, S, H, Hkv, seed=S + H, scale=scale, **kw)
+
+
+@pytest.mark.parametrize("H,Hkv", [(8, 1), (6, 2), (16, 2), (5, 1)])
+def test_other_head_ratios(H, Hkv):
+    """8, 3 and 5 query heads per kv head: several head groups per kv head in dQ, more streams in dK / dV."""
+    run_case("llm/scatter", "scatter", 1, 900, H, Hkv, seed=H, group_num=3)
+    run_case("llm/window_sink", "window_sink", 1, 900, H, Hkv, seed=H + 1, window=130, n_sink=40)
