@@ -500,6 +500,8 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
       (rc = check_strides("odk", dks, B, S, Hkv)) || (rc = check_strides("odv", dvs, B, S, Hkv)))
     return rc;
   if (!ls) return fail(INTRA_ERR_INVALID, "lse strides pointer is null");
+  for (int i = 0; i < 3; ++i)
+    if (ls[i] < 0) return fail(INTRA_ERR_INVALID, "lse stride %d is negative", i);
   if (!isfinite(scale)) return fail(INTRA_ERR_INVALID, "softmax_scale must be finite");
   if (scale == 0.f) return fail(INTRA_ERR_UNSUPPORTED, "backward: softmax_scale must not be zero");
   const int64_t* all[] = {qs, ks, vs, dos};

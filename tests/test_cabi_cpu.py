@@ -240,6 +240,7 @@ def test_bwd_validates_before_touching_the_gpu(lib):
     odd = _lib._i64x3(512 * 4 * 128, 4 * 128 + 4, 128)
     assert call(strides=(st,) * 4 + (odd,) + (st,) * 3) == _lib.INTRA_ERR_INVALID and "dout" in _lib.last_error()
     assert call(scale=float("nan")) == _lib.INTRA_ERR_INVALID
+    assert call(lse_strides=_lib._i64x3(4 * 512, -512, 1)) == _lib.INTRA_ERR_INVALID and "lse stride" in _lib.last_error()
     assert call(H=6, Hkv=4) == _lib.INTRA_ERR_INVALID
     assert call(pattern=7) == _lib.INTRA_ERR_INVALID
     assert call(scale=0.0) == _lib.INTRA_ERR_UNSUPPORTED
