@@ -302,7 +302,8 @@ struct LaunchMap {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-int check_strides(const char* name, const int64_t* st, int B, int S, int heads) {
+// `written`: the tensor is an output, so batch entries may not alias either
+int check_strides(const char* name, const int64_t* st, int B, int S, int heads, bool written = false) {
   if (!st) return fail(INTRA_ERR_INVALID, "%s strides pointer is null", name);
   for (int i = 0; i < 3; ++i) {
     if (st[i] < 0) return fail(INTRA_ERR_INVALID, "%s stride %d is negative", name, i);
@@ -310,7 +311,7 @@ int check_strides(const char* name, const int64_t* st, int B, int S, int heads) 
       return fail(INTRA_ERR_INVALID, "%s stride %d (%lld elements) breaks 16-byte alignment", name, i,
                   (long long)st[i]);
   }
-  if ((S > 1 && st[1] == 0) || (heads > 1 && st[2] == 0) || (B > 1 && st[0] == 0 && name[0] == 'o'))
+  if ((S > 1 && st[1] == 0) || (heads > 1 && st[2] == 0) || (B > 1 && st[0] == 0 && written))
     return fail(INTRA_ERR_INVALID, "%s has a zero stride over a dimension larger than 1", name);
   return INTRA_OK;
 }
@@ -330,7 +331,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   if ((rc = check_strides("q", qs, B, S, H))) return rc;
   if ((rc = check_strides("k", ks, B, S, Hkv))) return rc;
   if ((rc = check_strides("v", vs, B, S, Hkv))) return rc;
-  if ((rc = check_strides("o", os, B, S, H))) return rc;
+  if ((rc = check_strides("o", os, B, S, H, true))) return rc;
   if (!isfinite(scale)) return fail(INTRA_ERR_INVALID, "softmax_scale must be finite");
   if (want_lse) {
     if (!lse) return fail(INTRA_ERR_INVALID, "lse must be a non-null device pointer");
@@ -496,8 +497,8 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
   if (!dsum || !aligned16(dsum)) return fail(INTRA_ERR_INVALID, "the workspace must be a non-null, 16-byte aligned device pointer");
   if ((rc = check_strides("q", qs, B, S, H)) || (rc = check_strides("k", ks, B, S, Hkv)) ||
       (rc = check_strides("v", vs, B, S, Hkv)) || (rc = check_strides("o", os, B, S, H)) ||
-      (rc = check_strides("dout", dos, B, S, H)) || (rc = check_strides("odq", dqs, B, S, H)) ||
-      (rc = check_strides("odk", dks, B, S, Hkv)) || (rc = check_strides("odv", dvs, B, S, Hkv)))
+      (rc = check_strides("dout", dos, B, S, H)) || (rc = check_strides("dq", dqs, B, S, H, true)) ||
+      (rc = check_strides("dk", dks, B, S, Hkv, true)) || (rc = check_strides("dv", dvs, B, S, Hkv, true)))
     return rc;
   if (!ls) return fail(INTRA_ERR_INVALID, "lse strides pointer is null");
   for (int i = 0; i < 3; ++i)
