@@ -129,6 +129,7 @@ def test_configuration_errors():
         intra_attention_forward(model.layers[0].self_attn, q, k, k)
 
 
+@pytest.mark.timeout(600)  # the first import of transformers on a fresh machine takes a while
 def test_transformers_llama_model_trains_through_the_kernels():
     """A randomly initialised transformers LLaMA (tiny: 4 layers, 4 query / 2 kv heads of dim 128,
     rotary embeddings, RMSNorm, MLP - the real modelling code) with attn_implementation="intra":
