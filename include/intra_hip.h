@@ -128,11 +128,29 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
                   const int64_t lse_strides[3], int pattern, int group_num, int window, int block,
                   int offset, int n_sink, float softmax_scale, void* hip_stream);
 /* Floats of workspace that intra_llm_bwd needs for such a call (B*H*S rounded up to 4, plus with
- * sinks chunks * B * Hkv * min(n_sink, S) * 128, the queries being cut into chunks of 128 to
- * 1024 so that the sink pass fills the GPU); -1 if the request is invalid or unsupported
+ * sinks chunks * B * Hkv * min(n_sink, S) * 128, the queries being cut into chunks so that the
+ * sink pass has about one workgroup per CU); -1 if the request is invalid or unsupported
  * (intra_last_error() says why).  No counterpart in the reference. */
 int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int group_num,
                                 int window, int block, int offset, int n_sink);
+
+/* The same for intra_image_fwd: dq, dk, dv of image Scatter and Gather 0 (arguments as in
+ * intra_llm_bwd; pattern, width, text_len as in intra_image_fwd).  dq in one launch; the grid keys'
+ * dk / dv against the queries that see them (Scatter: their group's; Gather 0: the query patches
+ * around them, then their group's text queries added to the rows already written, both rounded to
+ * bf16); the text keys' dk / dv against all queries in chunks, as the sink keys of intra_llm_bwd.
+ * No counterpart in the reference (its FLUX training differentiates masked SDPA,
+ * experiments/flux/intra_processor.py:138-142). */
+int intra_image_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse,
+                    const void* dout, void* dq, void* dk, void* dv, float* workspace, int B, int S,
+                    int H, int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                    const int64_t v_strides[3], const int64_t o_strides[3],
+                    const int64_t dout_strides[3], const int64_t dq_strides[3],
+                    const int64_t dk_strides[3], const int64_t dv_strides[3],
+                    const int64_t lse_strides[3], int pattern, int width, int text_len,
+                    float softmax_scale, void* hip_stream);
+int64_t intra_image_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int width,
+                                  int text_len);
 
 /* ------------------------------------------------------------------ host-only helpers (no GPU)
  * How a call would be launched; mirrors the grid / per-set length derivation of the reference
@@ -173,6 +191,7 @@ int intra_model_mask_llm_ex(int pattern, int S, int group_num, int window, int b
  * dense mask. */
 int intra_model_mask_llm_bwd(int pattern, int S, int group_num, int window, int block, int offset,
                              int n_sink, uint8_t* count);
+int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint8_t* count);
 
 #ifdef __cplusplus
 }

@@ -32,8 +32,12 @@ SYMBOLS = {
                                                ctypes.POINTER(ctypes.c_int64)]),
     "intra_llm_bwd": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 9 +
                       [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_void_p]),
+    "intra_image_bwd": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 9 +
+                        [ctypes.c_int] * 3 + [ctypes.c_float, ctypes.c_void_p]),
+    "intra_image_bwd_workspace": (ctypes.c_int64, [ctypes.c_int] * 7),
     "intra_llm_bwd_workspace": (ctypes.c_int64, [ctypes.c_int] * 10),
     "intra_model_mask_llm_bwd": (ctypes.c_int, [ctypes.c_int] * 7 + [ctypes.c_void_p]),
+    "intra_model_mask_image_bwd": (ctypes.c_int, [ctypes.c_int] * 4 + [ctypes.c_void_p]),
     "intra_plan_llm_ex": (ctypes.c_int, [ctypes.c_int] * 10 + [ctypes.POINTER(IntraPlan)]),
     "intra_model_mask_llm_ex": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.c_void_p]),
     "intra_last_error": (ctypes.c_char_p, []),

@@ -15,7 +15,7 @@ import json
 import torch
 import torch.nn.functional as F
 
-from intra_amd import _lib, intra_image_attn, intra_llm_attn, intra_llm_attn_bwd
+from intra_amd import _lib, intra_image_attn, intra_image_attn_bwd, intra_llm_attn, intra_llm_attn_bwd
 from intra_amd.interface import TEXT_LEN
 
 PEAK_BF16_TFLOPS = 2516.6
@@ -181,6 +181,15 @@ def bench_image(args):
             ms = median_ms(lambda: intra_image_attn(q, k, v, pattern, width), args.warmup, args.iters)
             put(r, pattern, ms, pairs(1, pid, B, S, H, H, width, TEXT_LEN), B, H)
         r["interleaved_mean"] = round((r["scatter"] + r["gather0"]) / 2, 4)  # layers alternate the two patterns
+        if args.backward:
+            dout = qkv(B, S, H, H, seed=1)[0]
+            for pattern, pid in (("scatter", 0), ("gather0", 4)):
+                out, lse = intra_image_attn(q, k, v, pattern, width, return_lse=True)
+                ms = median_ms(lambda: intra_image_attn_bwd(q, k, v, out, lse, dout, pattern, width), args.warmup, args.iters)
+                tf = 10 * 128 * pairs(1, pid, B, S, H, H, width, TEXT_LEN) * H * B / (ms * 1e-3) / 1e12
+                r[pattern + "_bwd"] = round(ms, 4)
+                r[pattern + "_bwd_tflops"] = round(tf, 1)
+                r[pattern + "_bwd_pct_peak"] = round(100 * tf / PEAK_BF16_TFLOPS, 1)
         rows.append(r)
         print(json.dumps(r), flush=True)
     return rows
@@ -200,7 +209,7 @@ def main():
     p.add_argument("--dense", action="store_true", help="also time torch SDPA on the dense problem")
     p.add_argument("--model-patterns", action="store_true",
                    help="llm: also time block Scatter and window-with-sinks layers (g2s4 model setting)")
-    p.add_argument("--backward", action="store_true", help="llm: also time the backward pass (dq, dk, dv) of each pattern")
+    p.add_argument("--backward", action="store_true", help="also time the backward pass (dq, dk, dv) of each pattern")
     p.add_argument("--out", help="optional JSON output path")
     args = p.parse_args()
     args.seqlens = [int(x) for x in args.seqlens.split(",")]

@@ -43,8 +43,7 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   r->H = H;
   r->Hkv = Hkv;
   r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1, 64, 0, 0};  // derived fields: geom_finish() in shape_for()
-  // sink pass of the backward: about 512 workgroups, 128..1024 queries each
-  r->geom.sink_chunk = (int)std::min<int64_t>(1024, std::max<int64_t>(128, 64 * (((int64_t)S * B * Hkv + 512 * 64 - 1) / (512 * 64))));
+  r->geom.sink_chunk = 1024;  // backward: set by leading_chunk() once the number of leading keys is known
   if (domain == 0) {
     if (!extended && (pattern == INTRA_LLM_BLOCK_SCATTER || pattern == INTRA_LLM_WINDOW_SINK))
       return fail(INTRA_ERR_INVALID, "unknown LLM pattern id %d (0 scatter, 1 gather1, 4 window)", pattern);
@@ -438,10 +437,19 @@ int run_bwd_keys(const intra::BParams& p, hipStream_t stream) {
   return run_bwd_keys_mode<R, false, intra::BWD_DV>(p, stream);
 }
 
-// The sink rows of dk and dv: partial sums per chunk of queries, then their sum (twice, dk and dv
-// share the partial buffer; everything is ordered by the stream).
-int run_bwd_sinks(const intra::BParams& p, hipStream_t stream) {
-  using R = intra::KeyRowsSinks;
+// Queries per workgroup of the pass over the `ns` leading keys (LLM sinks, image text keys): about
+// one workgroup per CU, at least 128 queries each, a multiple of 64.
+int leading_chunk(int S, int B, int Hkv, int ns) {
+  const int64_t row_wgs = (int64_t)B * Hkv * ((ns + 255) / 256);
+  int64_t chunks = std::max<int64_t>(1, (256 + row_wgs - 1) / row_wgs);
+  chunks = std::min<int64_t>(chunks, std::max(1, S / 128));
+  return (int)(64 * ((S + 64 * chunks - 1) / (64 * chunks)));
+}
+
+// The rows of dk and dv of the leading keys: partial sums per chunk of queries, then their sum
+// (twice: dk and dv share the partial buffer; everything is ordered by the stream).
+template <class R>
+int run_bwd_leading(const intra::BParams& p, hipStream_t stream) {
   const int ns = R::max_rows(p.geom), chunks = R::num_sets(p.geom);
   const int64_t threads = (int64_t)p.B * p.Hkv * ns * 32;
   const unsigned blocks = (unsigned)((threads + 255) / 256);
@@ -461,13 +469,22 @@ int run_bwd_sinks(const intra::BParams& p, hipStream_t stream) {
   return INTRA_OK;
 }
 
-// floats of workspace: D = rowsum(dO o O) per (batch, head, token), then the partial sums of the sink pass
+// keys every query sees, handled by run_bwd_leading
+int leading_keys(const Request& r) {
+  if (r.kind == KIND_LLM_BLOCK_SCATTER || r.kind == KIND_LLM_WINDOW_SINK) return std::min(r.geom.ns, r.S);
+  if (r.kind == KIND_IMG_SCATTER || r.kind == KIND_IMG_GATHER0) return r.geom.text_len;
+  return 0;
+}
+
+// floats of workspace: D = rowsum(dO o O) per (batch, head, token), then the partial sums of the leading keys
 int64_t bwd_dsum_floats(int B, int S, int H) { return ((int64_t)B * H * S + 3) & ~(int64_t)3; }
 int64_t bwd_workspace_floats(const Request& r) {
   int64_t n = bwd_dsum_floats(r.B, r.S, r.H);
-  const int ns = std::min(r.geom.ns, r.S);
-  if ((r.kind == KIND_LLM_BLOCK_SCATTER || r.kind == KIND_LLM_WINDOW_SINK) && ns > 0)
-    n += (int64_t)((r.S + r.geom.sink_chunk - 1) / r.geom.sink_chunk) * r.B * r.Hkv * ns * 128;
+  const int ns = leading_keys(r);
+  if (ns > 0) {
+    const int chunk = leading_chunk(r.S, r.B, r.Hkv, ns);
+    n += (int64_t)((r.S + chunk - 1) / chunk) * r.B * r.Hkv * ns * 128;
+  }
   return n;
 }
 
@@ -478,14 +495,14 @@ int bwd_supported(const Request& r) {
   return INTRA_OK;
 }
 
-int run_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
+int run_bwd(int domain, const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
             void* dq, void* dk, void* dv, float* dsum, int B, int S, int H, int Hkv, const int64_t* qs,
             const int64_t* ks, const int64_t* vs, const int64_t* os, const int64_t* dos, const int64_t* dqs,
             const int64_t* dks, const int64_t* dvs, const int64_t* ls, int pattern, int group_num, int window,
             int block, int offset, int n_sink, float scale, void* stream) {
   g_err[0] = 0;
   Request r;
-  int rc = make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true);
+  int rc = make_request(domain, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, domain == 0);
   if (rc) return rc;
   if ((rc = bwd_supported(r))) return rc;
   const void* ins[] = {q, k, v, o, dout, dq, dk, dv};
@@ -537,6 +554,11 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
   Shape sh;
   if (!shape_for(r, default_hp(H / Hkv), &sh)) return fail(INTRA_ERR_UNSUPPORTED, "no kernel shape for this request");
   p.geom = sh.geom;
+  const int ns = leading_keys(r);
+  if (ns > 0) {
+    p.geom.ns = ns;
+    p.geom.sink_chunk = leading_chunk(S, B, Hkv, ns);
+  }
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (sh.map) {
     case MAP_LLM_SCATTER:
@@ -551,14 +573,22 @@ int run_bwd(const void* q, const void* k, const void* v, const void* o, const fl
     case MAP_LLM_BLOCK_SCATTER:
       if ((rc = run_bwd_dq<MapLlmBlockScatter>(p, sh.hp, st))) return rc;
       if ((rc = run_bwd_keys<intra::KeyRowsBlockScatter>(p, st))) return rc;
-      break;
+      return ns > 0 ? run_bwd_leading<intra::KeyRowsSinks>(p, st) : INTRA_OK;
     case MAP_LLM_WINDOW_SINK:
       if ((rc = run_bwd_dq<MapLlmWindowSink>(p, sh.hp, st))) return rc;
       if ((rc = run_bwd_keys<intra::KeyRowsWindowSink>(p, st))) return rc;
-      break;
+      return ns > 0 ? run_bwd_leading<intra::KeyRowsSinks>(p, st) : INTRA_OK;
+    case MAP_IMG_SCATTER:  // grid keys against their group's queries, text keys against all queries
+      if ((rc = run_bwd_dq<MapImgScatter>(p, sh.hp, st))) return rc;
+      if ((rc = run_bwd_keys<intra::KeyRowsImgGroup<false>>(p, st))) return rc;
+      return run_bwd_leading<intra::KeyRowsText>(p, st);
+    case MAP_IMG_GATHER0:  // grid keys against the grid queries around them, plus their group's text queries
+      if ((rc = run_bwd_dq<MapImgGather0>(p, sh.hp, st))) return rc;
+      if ((rc = run_bwd_keys<intra::KeyRowsImgWindow>(p, st))) return rc;
+      if ((rc = run_bwd_keys<intra::KeyRowsImgGroup<true>>(p, st))) return rc;
+      return run_bwd_leading<intra::KeyRowsText>(p, st);
     default: return fail(INTRA_ERR_UNSUPPORTED, "backward: no kernels for this pattern");
   }
-  return std::min(r.geom.ns, r.S) > 0 ? run_bwd_sinks(p, st) : INTRA_OK;
 }
 
 // Host walk of the backward decomposition: count[q * S + k] += 1 for every (query, key) pair that
@@ -573,9 +603,10 @@ void bwd_walk(const IntraGeom& ge, uint8_t* count) {
       for (int t = r0; t <= r1; ++t) {
         const int kp = m.row_pos(t);
         if (!m.store(kp)) continue;
-        const int lo = m.lo(t), hi = std::min(m.hi(t), m.n_cols() - 1);
-        for (int c = std::max(lo, m.block_lo(r0, r1)); c <= std::min(hi, m.block_hi(r0, r1)); ++c)
-          ++count[(size_t)m.col_pos(c) * S + kp];
+        const int lo = std::max(m.lo(t), m.block_lo(r0, r1));
+        const int hi = std::min(std::min(m.hi(t), m.n_cols() - 1), m.block_hi(r0, r1));
+        for (int c = lo; c <= hi; ++c)
+          if (!R::kBlockPredicate || m.sees(t, c & ~31)) ++count[(size_t)m.col_pos(c) * S + kp];
       }
     }
 }
@@ -592,8 +623,10 @@ int model_mask_bwd(const Request& r, uint8_t* count) {
     case MAP_LLM_WINDOW_SINK: bwd_walk<intra::KeyRowsWindowSink>(sh.geom, count); break;
     default: return fail(INTRA_ERR_UNSUPPORTED, "backward: no kernels for this pattern");
   }
-  if (std::min(r.geom.ns, r.S) > 0 && (sh.map == MAP_LLM_BLOCK_SCATTER || sh.map == MAP_LLM_WINDOW_SINK))
+  if (leading_keys(r) > 0) {
+    sh.geom.sink_chunk = leading_chunk(r.S, 1, 1, leading_keys(r));
     bwd_walk<intra::KeyRowsSinks>(sh.geom, count);
+  }
   return INTRA_OK;
 }
 
@@ -605,6 +638,22 @@ int model_mask(const Request& r, int heads_per_block, int waves, uint8_t* count)
   if (!shape_for(r, hp, &ph))
     return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
   by_map<ModelWalk>(ph.map, ph.geom, ph.hp, ph.nw, count);
+  return INTRA_OK;
+}
+
+int model_mask_image_bwd(const Request& r, uint8_t* count) {
+  Shape sh;
+  if (!shape_for(r, 1, &sh)) return fail(INTRA_ERR_UNSUPPORTED, "no kernel shape for this request");
+  IntraGeom ge = sh.geom;
+  ge.ns = ge.text_len;  // the text keys are the leading keys every query sees
+  ge.sink_chunk = leading_chunk(r.S, 1, 1, ge.ns);
+  if (r.kind == KIND_IMG_SCATTER) {
+    bwd_walk<intra::KeyRowsImgGroup<false>>(ge, count);
+  } else {
+    bwd_walk<intra::KeyRowsImgWindow>(ge, count);
+    bwd_walk<intra::KeyRowsImgGroup<true>>(ge, count);
+  }
+  bwd_walk<intra::KeyRowsText>(ge, count);
   return INTRA_OK;
 }
 
@@ -653,7 +702,7 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
                   const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[3],
                   int pattern, int group_num, int window, int block, int offset, int n_sink,
                   float softmax_scale, void* hip_stream) {
-  return run_bwd(q, k, v, o, lse, dout, dq, dk, dv, workspace, B, S, H, Hkv, q_strides, k_strides, v_strides,
+  return run_bwd(0, q, k, v, o, lse, dout, dq, dk, dv, workspace, B, S, H, Hkv, q_strides, k_strides, v_strides,
                  o_strides, dout_strides, dq_strides, dk_strides, dv_strides, lse_strides, pattern, group_num,
                  window, block, offset, n_sink, softmax_scale, hip_stream);
 }
@@ -667,6 +716,24 @@ int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int g
   return bwd_workspace_floats(r);
 }
 
+int intra_image_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
+                    void* dq, void* dk, void* dv, float* workspace, int B, int S, int H, int Hkv,
+                    const int64_t q_strides[3], const int64_t k_strides[3], const int64_t v_strides[3],
+                    const int64_t o_strides[3], const int64_t dout_strides[3], const int64_t dq_strides[3],
+                    const int64_t dk_strides[3], const int64_t dv_strides[3], const int64_t lse_strides[3],
+                    int pattern, int width, int text_len, float softmax_scale, void* hip_stream) {
+  return run_bwd(1, q, k, v, o, lse, dout, dq, dk, dv, workspace, B, S, H, Hkv, q_strides, k_strides, v_strides,
+                 o_strides, dout_strides, dq_strides, dk_strides, dv_strides, lse_strides, pattern, width, text_len,
+                 0, 0, 0, softmax_scale, hip_stream);
+}
+
+int64_t intra_image_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int width, int text_len) {
+  g_err[0] = 0;
+  Request r;
+  if (make_request(1, pattern, B, S, H, Hkv, width, text_len, &r)) return -1;
+  return bwd_workspace_floats(r);
+}
+
 int intra_model_mask_llm_bwd(int pattern, int S, int group_num, int window, int block, int offset, int n_sink,
                              uint8_t* count) {
   g_err[0] = 0;
@@ -675,6 +742,15 @@ int intra_model_mask_llm_bwd(int pattern, int S, int group_num, int window, int 
   int rc = make_request(0, pattern, 1, S, 1, 1, group_num, window, &r, block, offset, n_sink, true);
   if (rc) return rc;
   return model_mask_bwd(r, count);
+}
+
+int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint8_t* count) {
+  g_err[0] = 0;
+  if (!count) return fail(INTRA_ERR_INVALID, "count is null");
+  Request r;
+  int rc = make_request(1, pattern, 1, S, 1, 1, width, text_len, &r);
+  if (rc) return rc;
+  return model_mask_image_bwd(r, count);
 }
 
 const char* intra_last_error(void) { return g_err; }

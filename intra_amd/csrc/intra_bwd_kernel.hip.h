@@ -1,7 +1,7 @@
 // Backward kernels of the sparse attention for gfx950 (MI355X): dQ, dK and dV for the causal LLM
 // patterns (Scatter, Gather 1, 64-aligned window, block Scatter with stripe offsets and sinks,
-// per-token window with sinks).  Which rows meet which columns comes from the row maps of
-// intra_bwd_maps.h.
+// per-token window with sinks) and the image patterns (Scatter, Gather 0).  Which rows meet which
+// columns comes from the row maps of intra_bwd_maps.h.
 //
 // The reference has no backward kernels (its README names them as missing; training there runs
 // through masked SDPA / FlexAttention, experiments/llm/llama_intra.py:26).  The math is the usual
@@ -312,7 +312,18 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
         continue;
       }
       const int sb_lo = cb + 32 * jb;  // first column of the block
-      const bool masked = !block_unmasked(wb, kpre, sb_lo);
+      // maps with a block predicate: a row meets the whole block or nothing of it
+      bool lane_sees = true;
+      uint64_t seeing = ~0ull;
+      if (RMAP::kBlockPredicate) {
+        lane_sees = map.sees(row, sb_lo);
+        seeing = __builtin_amdgcn_ballot_w64(lane_sees);
+        if (seeing == 0) {
+          have = false;
+          continue;
+        }
+      }
+      const bool masked = RMAP::kBlockPredicate ? seeing != ~0ull : !block_unmasked(wb, kpre, sb_lo);
       // this block, the one that follows in this order, and the one after that
       const int c1off = slot0 + blk * BLOCK32, c2off = c1off + TILE_BYTES;
       const int c1n = blk == 0 ? c1off + BLOCK32 : slot1, c2n = c1n + TILE_BYTES;
@@ -342,8 +353,11 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
       const float* sc = reinterpret_cast<const float*>(smem + slot0 + 2 * TILE_BYTES) + 32 * blk + 4 * h32;
       if (masked) {  // scores of invisible pairs become -inf (for a positive scale): weight 0
 #pragma unroll
-        for (int e = 0; e < 16; ++e)
-          if (!key_visible(sb_lo + 8 * (e >> 2) + 4 * h32 + (e & 3), kpre, lo_l, hi_l)) s_cur[e] = s_hidden;
+        for (int e = 0; e < 16; ++e) {
+          const bool vis = RMAP::kBlockPredicate ? lane_sees
+                                                 : key_visible(sb_lo + 8 * (e >> 2) + 4 * h32 + (e & 3), kpre, lo_l, hi_l);
+          if (!vis) s_cur[e] = s_hidden;
+        }
       }
       floatx16 dp, s_next;
       bf16x8 wp[2];
@@ -434,6 +448,15 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
       auto q1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
       if (keep) {
         u32x4 pk = {q0[0], q1[0], q0[1], q1[1]};
+        if (RMAP::kAccumulate) {  // add to what an earlier pass has written (both rounded to bf16)
+          const u32x4 old = *reinterpret_cast<const u32x4*>(orow + 32 * db + 16 * g2);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            floatx2 s2 = {__uint_as_float(pk[i] << 16) + __uint_as_float(old[i] << 16),
+                          __uint_as_float(pk[i] & 0xffff0000u) + __uint_as_float(old[i] & 0xffff0000u)};
+            pk[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(s2, bf16x2));
+          }
+        }
         *reinterpret_cast<u32x4*>(orow + 32 * db + 16 * g2) = pk;
       }
     }

@@ -139,29 +139,10 @@ def intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", group_num=8, 
         raise ValueError(f"unknown pattern {pattern!r}")
     if pattern == "gather1" and (group_num != 8 or q.shape[1] % (group_num * group_num)):
         raise ValueError(f"gather1 needs group_num=8 and seqlen % 64 == 0, got G={group_num}, S={q.shape[1]}")
-    fix = lambda t: t if (t.stride(-1) == 1 and _aligned(t)) else t.contiguous()
-    out, dout = fix(out), fix(dout)
-    if out.shape != q.shape or dout.shape != q.shape or out.dtype != q.dtype or dout.dtype != q.dtype:
-        raise ValueError("out and dout must have the shape and dtype of q")
     B, S, H, _ = q.shape
-    if lse.shape != (B, H, S) or lse.dtype != torch.float32:
-        raise ValueError("lse must be the (batch, heads, seqlen) fp32 tensor of the forward call")
     args = (ids[pattern], int(group_num), int(window), int(block), int(offset), int(n_sink))
     n_work = _C.intra_llm_bwd_workspace(B, S, H, k.shape[2], *args)
-    if n_work < 0:
-        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
-    dq, dk, dv = (torch.empty(t.shape, dtype=t.dtype, device=t.device) for t in (q, k, v))
-    work = torch.empty(n_work, dtype=torch.float32, device=q.device)
-    guard, stream = _stream_on(q.device)
-    with guard:
-        rc = _C.intra_llm_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), dout.data_ptr(),
-                              dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), work.data_ptr(), B, S, H, k.shape[2],
-                              _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
-                              _lib.strides3(dout), _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv),
-                              _lib.strides3(lse), *args, float(_scale(q, softmax_scale)), stream)
-    if rc != _lib.INTRA_OK:
-        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
-    return dq, dk, dv
+    return _bwd_call(_C.intra_llm_bwd, n_work, q, k, v, out, lse, dout, args, _scale(q, softmax_scale))
 
 
 class _LlmAttnFunction(torch.autograd.Function):
@@ -184,6 +165,64 @@ def intra_llm_attn_func(q, k, v, pattern="scatter", group_num=8, window=576, sof
                         n_sink=0):
     """intra_llm_attn as a differentiable function (torch.autograd): forward and backward kernels."""
     return _LlmAttnFunction.apply(q, k, v, pattern, group_num, window, softmax_scale, block, offset, n_sink)
+
+
+def _bwd_call(fn, n_work, q, k, v, out, lse, dout, args, scale):
+    """Shared part of the backward wrappers: checks, allocation of the results and the workspace, the call."""
+    fix = lambda t: t if (t.stride(-1) == 1 and _aligned(t)) else t.contiguous()
+    out, dout = fix(out), fix(dout)
+    if out.shape != q.shape or dout.shape != q.shape or out.dtype != q.dtype or dout.dtype != q.dtype:
+        raise ValueError("out and dout must have the shape and dtype of q")
+    B, S, H, _ = q.shape
+    if lse.shape != (B, H, S) or lse.dtype != torch.float32:
+        raise ValueError("lse must be the (batch, heads, seqlen) fp32 tensor of the forward call")
+    if n_work < 0:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
+    dq, dk, dv = (torch.empty(t.shape, dtype=t.dtype, device=t.device) for t in (q, k, v))
+    work = torch.empty(n_work, dtype=torch.float32, device=q.device)
+    guard, stream = _stream_on(q.device)
+    with guard:
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), dout.data_ptr(),
+                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), work.data_ptr(), B, S, H, k.shape[2],
+                _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out), _lib.strides3(dout),
+                _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv), _lib.strides3(lse), *args, float(scale), stream)
+    if rc != _lib.INTRA_OK:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
+    return dq, dk, dv
+
+
+def intra_image_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", width=64, softmax_scale=None):
+    """Gradients (dq, dk, dv) of intra_image_attn, given the forward results `out`, `lse`
+    (return_lse=True) and the gradient `dout` of `out`.  The reference has no backward kernels (its
+    FLUX training differentiates masked SDPA, experiments/flux/intra_processor.py:138-142)."""
+    q, k, v = _check(q, k, v)
+    if width not in (64, 128):
+        raise ValueError("image kernels are compiled for width 64 and 128")
+    if q.shape[1] != TEXT_LEN + width * width:
+        raise ValueError(f"expected {TEXT_LEN} text + {width}x{width} image tokens, got {q.shape[1]}")
+    B, S, H, _ = q.shape
+    args = (IMAGE_PATTERNS[pattern], int(width), TEXT_LEN)
+    n_work = _C.intra_image_bwd_workspace(B, S, H, k.shape[2], *args)
+    return _bwd_call(_C.intra_image_bwd, n_work, q, k, v, out, lse, dout, args, _scale(q, softmax_scale))
+
+
+class _ImageAttnFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q, k, v, pattern, width, softmax_scale):
+        out, lse = intra_image_attn(q, k, v, pattern, width, softmax_scale, return_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.args = (pattern, width, softmax_scale)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        return intra_image_attn_bwd(q, k, v, out, lse, dout, *ctx.args) + (None,) * 3
+
+
+def intra_image_attn_func(q, k, v, pattern="scatter", width=64, softmax_scale=None):
+    """intra_image_attn as a differentiable function (torch.autograd): forward and backward kernels."""
+    return _ImageAttnFunction.apply(q, k, v, pattern, width, softmax_scale)
 
 
 def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None, return_lse=False):

@@ -250,16 +250,29 @@ def test_bwd_validates_before_touching_the_gpu(lib):
     assert call(ptrs=(P,) * 9 + (P + 4,)) == _lib.INTRA_ERR_INVALID and "workspace" in _lib.last_error()
 
 
+def _leading_chunks(S, B, Hkv, ns):
+    """The library's rule for the pass over leading keys: about one workgroup per CU, chunks of at
+    least 128 queries and a multiple of 64."""
+    row_wgs = B * Hkv * -(-ns // 256)
+    chunks = min(max(1, -(-256 // row_wgs)), max(1, S // 128))
+    chunk = 64 * -(-S // (64 * chunks))
+    return -(-S // chunk)
+
+
 def test_bwd_workspace_size(lib):
     assert lib.intra_llm_bwd_workspace(1, 1000, 8, 2, 0, 8, 576, 256, 0, 0) == 8000
     assert lib.intra_llm_bwd_workspace(2, 1001, 3, 3, 4, 8, 576, 256, 0, 0) == 6008  # rounded up to 4
-    # sinks: chunks x B x Hkv x n_sink x 128 more; chunks of 128 queries here (64 * ceil(S*B*Hkv / 32768), at least 128)
-    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 24000 + 24 * 2 * 64 * 128
-    # ... of 1024 queries for long sequences
-    assert lib.intra_llm_bwd_workspace(1, 65536, 32, 8, 9, 2, 575, 256, 0, 64) == 65536 * 32 + 64 * 8 * 64 * 128
+    # sinks: chunks x B x Hkv x n_sink x 128 more
+    assert _leading_chunks(3000, 1, 2, 64) == 16 and _leading_chunks(65536, 1, 8, 64) == 32
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 24000 + 16 * 2 * 64 * 128
+    assert lib.intra_llm_bwd_workspace(1, 65536, 32, 8, 9, 2, 575, 256, 0, 64) == 65536 * 32 + 32 * 8 * 64 * 128
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 256, 1, 0) == 24000
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 128, 1, 0) == -1
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 3, 0, 8, 576, 256, 0, 0) == -1
+    # image patterns: the 512 text keys are the leading keys
+    S = 512 + 64 * 64
+    assert lib.intra_image_bwd_workspace(1, S, 24, 24, 0, 64, 512) == S * 24 + _leading_chunks(S, 1, 24, 512) * 24 * 512 * 128
+    assert lib.intra_image_bwd_workspace(1, S, 24, 24, 4, 64, 511) == -1
 
 
 BWD_CASES = [
@@ -286,4 +299,17 @@ def test_backward_key_row_maps_equal_mask(lib, pattern, kind, S, kw):
                                       kw.get("offset", 0), kw.get("n_sink", 0), count.ctypes.data)
     assert rc == 0, _lib.last_error()
     want = oracle.mask_rows(kind, S, **kw).numpy().astype(np.uint8)
+    assert np.array_equal(count, want), np.argwhere(count != want)[:5]
+
+
+@pytest.mark.parametrize("W,T", [(64, 512), (16, 8), (24, 72), (40, 200), (32, 96), (48, 64)])
+@pytest.mark.parametrize("kind,pattern", [("image/scatter", 0), ("image/gather0", 4)])
+def test_backward_key_row_maps_equal_mask_image(lib, W, T, kind, pattern):
+    """The dk / dv passes of the image patterns (grid keys by group or by window, text queries'
+    share, text keys against all queries) multiply every pair of the mask exactly once."""
+    S = T + W * W
+    count = np.zeros((S, S), dtype=np.uint8)
+    rc = lib.intra_model_mask_image_bwd(pattern, S, W, T, count.ctypes.data)
+    assert rc == 0, _lib.last_error()
+    want = oracle.mask_rows(kind, S, width=W, text_len=T).numpy().astype(np.uint8)
     assert np.array_equal(count, want), np.argwhere(count != want)[:5]
