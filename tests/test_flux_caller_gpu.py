@@ -19,7 +19,7 @@ import torch
 import torch.nn.functional as F
 
 import oracle
-from intra_amd import intra_image_attn
+from intra_amd import intra_image_attn, intra_image_attn_func
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -67,7 +67,8 @@ def joint_layer(attn, hidden, text, pattern, width, use_kernel):
     if use_kernel:
         qv, kv, vv = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
         assert qv.stride(2) == q.shape[2] * D and qv.stride(1) == D  # (B, H, S, D) storage
-        a = intra_image_attn(qv, kv, vv, pattern=pattern, width=width, softmax_scale=scale).transpose(1, 2)
+        attend = intra_image_attn_func if torch.is_grad_enabled() else intra_image_attn  # training / inference
+        a = attend(qv, kv, vv, pattern=pattern, width=width, softmax_scale=scale).transpose(1, 2)
     else:
         mask = oracle.mask_rows(f"image/{pattern}", q.shape[2], device=q.device, width=width)
         a = F.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=mask, scale=scale).to(q.dtype)
@@ -96,3 +97,28 @@ def test_flux_style_layers_kernel_equals_masked_sdpa(width, heads, batch):
             # feed the kernel path's result forward, as the model would (residual + normalise)
             hidden = F.layer_norm((hidden.float() + h_k.float()), (dim,)).to(torch.bfloat16)
             text = F.layer_norm((text.float() + t_k.float()), (dim,)).to(torch.bfloat16)
+
+
+@pytest.mark.parametrize("pattern", ["scatter", "gather0"])
+def test_flux_style_layer_trains_through_the_kernels(pattern):
+    """The branch of the processor that needs gradients (intra_processor.py:138-142, masked SDPA in
+    the reference) on the backward kernels: gradients of the layer's weights and inputs against
+    the masked-SDPA path, for the distillation-style loss the reference trains with (a mean squared
+    error on the layer outputs).  Tolerance: relative l2 error 3e-2 per tensor (the SDPA path runs
+    its attention in fp32, the kernels in bf16 with fp32 accumulation)."""
+    width, heads, batch = 64, 2, 1
+    dim = heads * 128
+    g = torch.Generator().manual_seed(7)
+    hidden0 = torch.randn(batch, width * width, dim, generator=g).to(torch.bfloat16).to(DEV)
+    text0 = torch.randn(batch, TEXT, dim, generator=g).to(torch.bfloat16).to(DEV)
+    attn = JointAttention(dim, heads, seed=3).to(DEV).to(torch.bfloat16)
+    results = []
+    for use_kernel in (True, False):
+        hidden, text = hidden0.clone().requires_grad_(True), text0.clone().requires_grad_(True)
+        attn.zero_grad(set_to_none=True)
+        t_out, h_out, _ = joint_layer(attn, hidden, text, pattern, width, use_kernel=use_kernel)
+        (t_out.float().square().mean() + h_out.float().square().mean()).backward()
+        results.append([hidden.grad, text.grad] + [p.grad.clone() for p in attn.parameters()])
+    for i, (a, b) in enumerate(zip(*results)):
+        rel = ((a.float() - b.float()).norm() / b.float().norm()).item()
+        assert torch.isfinite(a).all() and rel <= 3e-2, (i, rel)
