@@ -123,3 +123,15 @@ def test_backward_block_scatter(lib, S, G, blk64, off, ns_frac):
     assert rc == 0, _lib.last_error()
     want = oracle.mask_rows("llm/block_scatter", S, group_num=G, block=blk, offset=off, n_sink=ns)
     assert torch.equal(count, want.to(torch.uint8))
+
+
+@settings(max_examples=60, deadline=None, suppress_health_check=[HealthCheck.function_scoped_fixture])
+@given(w8=st.integers(2, 9), t8=st.integers(1, 50), gather=st.booleans())
+def test_backward_image_patterns(lib, w8, t8, gather):
+    W, T = 8 * w8, 8 * t8
+    S = T + W * W
+    count = np.zeros((S, S), dtype=np.uint8)
+    rc = lib.intra_model_mask_image_bwd(4 if gather else 0, S, W, T, count.ctypes.data)
+    assert rc == 0, _lib.last_error()
+    kind = "image/gather0" if gather else "image/scatter"
+    assert torch.equal(torch.from_numpy(count), oracle.mask_rows(kind, S, width=W, text_len=T).to(torch.uint8))
