@@ -171,7 +171,7 @@ def bench_llm(args):
 def bench_image(args):
     rows = []
     B, H = args.batch, args.image_heads
-    for width in (64, 128):
+    for width in args.widths:
         S = TEXT_LEN + width * width
         q, k, v = qkv(B, S, H, H)
         r = {"width": width, "seqlen": S}
@@ -204,6 +204,7 @@ def main():
     p.add_argument("--heads", type=int, default=32)
     p.add_argument("--kv-heads", type=int, default=8)
     p.add_argument("--image-heads", type=int, default=24)
+    p.add_argument("--widths", default="64,128", help="image: latent grid sides (64: 1024 x 1024, 128: 2048 x 2048)")
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--iters", type=int, default=50)
     p.add_argument("--dense", action="store_true", help="also time torch SDPA on the dense problem")
@@ -213,6 +214,7 @@ def main():
     p.add_argument("--out", help="optional JSON output path")
     args = p.parse_args()
     args.seqlens = [int(x) for x in args.seqlens.split(",")]
+    args.widths = [int(x) for x in args.widths.split(",")]
     args.groups = [int(x) for x in args.groups.split(",")]
     print(f"device: {torch.cuda.get_device_name()}  torch {torch.__version__}  peak {PEAK_BF16_TFLOPS} TFLOP/s")
     rows = bench_llm(args) if args.mode == "llm" else bench_image(args)
