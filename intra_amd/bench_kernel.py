@@ -82,6 +82,18 @@ def bench_llm(args):
         if args.dense:
             ms = median_ms(lambda: dense_sdpa(q, k, v, True), args.warmup, args.iters)
             put(r, "dense", ms, S * (S + 1) // 2, B, H)
+        if args.cpu and S <= 8192:
+            # torch SDPA on the host cores for the dense causal problem, fp32: the scale of a CPU run
+            # beside the GPU rows (one warm-up, median of 3)
+            import time
+            qc, kc, vc = (x.float().cpu() for x in (q, k, v))
+            times = []
+            for _ in range(4):
+                t0 = time.perf_counter()
+                dense_sdpa(qc, kc, vc, True)
+                times.append((time.perf_counter() - t0) * 1e3)
+            r["dense_cpu_ms"] = round(sorted(times[1:])[1], 2)
+            r["cpu_cores"] = torch.get_num_threads()
         for G in args.groups:
             ms = median_ms(lambda: intra_llm_attn(q, k, v, "scatter", group_num=G), args.warmup, args.iters)
             put(r, f"scatter_g{G}", ms, pairs(0, 0, B, S, H, Hkv, G, 576), B, H)
@@ -208,6 +220,7 @@ def main():
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--iters", type=int, default=50)
     p.add_argument("--dense", action="store_true", help="also time torch SDPA on the dense problem")
+    p.add_argument("--cpu", action="store_true", help="llm: also time dense causal SDPA on the host CPU (S <= 8192)")
     p.add_argument("--model-patterns", action="store_true",
                    help="llm: also time block Scatter and window-with-sinks layers (g2s4 model setting)")
     p.add_argument("--backward", action="store_true", help="also time the backward pass (dq, dk, dv) of each pattern")
