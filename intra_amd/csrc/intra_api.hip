@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <algorithm>
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/intra_hip.h"
@@ -264,15 +266,15 @@ template <class MAP> struct ModelWalk {
 
 // One persistent workgroup per CU (LDS allows no more), in multiples of the 8 XCDs.
 int launch_grid(int work_items) {
-  static int cus[64] = {0};
+  static std::atomic<int> cus[64];  // CU count per device, 0 = not asked yet (same answer from every thread)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
-  if (cus[dev] == 0) {
-    int n = 0;
+  int n = cus[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return -1;
-    cus[dev] = n;
+    cus[dev].store(n, std::memory_order_relaxed);
   }
-  int g = (cus[dev] / 8) * 8;
+  int g = (n / 8) * 8;
   if (g < 8) g = 8;
   return work_items < g ? work_items : g;
 }
