@@ -443,7 +443,7 @@ int run_bwd_keys(const intra::BParams& p, hipStream_t stream) {
 // one workgroup per CU, at least 128 queries each, a multiple of 64.
 int leading_chunk(int S, int B, int Hkv, int ns) {
   const int64_t row_wgs = (int64_t)B * Hkv * ((ns + 255) / 256);
-  int64_t chunks = std::max<int64_t>(1, (256 + row_wgs - 1) / row_wgs);
+  int64_t chunks = std::max<int64_t>(1, 256 / row_wgs);  // at most one workgroup per CU: no second, thin round
   chunks = std::min<int64_t>(chunks, std::max(1, S / 128));
   return (int)(64 * ((S + 64 * chunks - 1) / (64 * chunks)));
 }

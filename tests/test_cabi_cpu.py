@@ -254,7 +254,7 @@ def _leading_chunks(S, B, Hkv, ns):
     """The library's rule for the pass over leading keys: about one workgroup per CU, chunks of at
     least 128 queries and a multiple of 64."""
     row_wgs = B * Hkv * -(-ns // 256)
-    chunks = min(max(1, -(-256 // row_wgs)), max(1, S // 128))
+    chunks = min(max(1, 256 // row_wgs), max(1, S // 128))
     chunk = 64 * -(-S // (64 * chunks))
     return -(-S // chunk)
 
