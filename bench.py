@@ -32,6 +32,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--seqlen", type=int, default=32768)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--softmax", choices=["auto", "exact", "fast"], default="auto",
+                    help="softmax arithmetic of the kernel (auto: what a plain call gets)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run three plain 1 GiB device copies, the known-size kernel that scales "
                          "FETCH_SIZE / WRITE_SIZE readings of a counter run")
@@ -43,10 +45,12 @@ def main():
     import torch
 
     import oracle
+    import intra_amd
     from intra_amd import _lib, intra_llm_attn
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     assert os.path.exists(_lib.LIB_PATH), "libintra_hip.so is not built"
+    intra_amd.set_softmax_mode(args.softmax)
     dev = torch.device("cuda:0")
     B, S, H, Hkv, G = 1, args.seqlen, 32, 8, 8
     g = torch.Generator(device="cpu").manual_seed(0)
@@ -105,7 +109,7 @@ def main():
         "ms_per_call": round(wall_ms, 4), "pct_of_peak": round(100 * tflops / PEAK_BF16_TFLOPS, 2),
         "kernel_ms": {"avg": round(kern_avg, 4), "median": round(kern_ms[len(kern_ms) // 2], 4),
                       "min": round(kern_ms[0], 4), "p90": round(kern_ms[int(0.9 * (len(kern_ms) - 1))], 4)},
-        "parity_max_abs_err": err,
+        "parity_max_abs_err": err, "softmax": args.softmax,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(S)},

@@ -100,8 +100,24 @@ int intra_llm_fwd_ex(const void* q, const void* k, const void* v, void* o, int B
  * TORCH_CHECK messages of flash_api.cpp. */
 const char* intra_last_error(void);
 
-/* Library version, major*10000 + minor*100 + patch. */
+/* Library version, major*10000 + minor*100 + patch (0.2.0). */
+#define INTRA_VERSION 200
 int intra_version(void);
+
+/* Softmax arithmetic of the forward entry points.  The reference scales the fp32 scores after the
+ * first product (csrc/flash_attn/src/softmax.h:65-91); so does the EXACT mode here.  FAST multiplies
+ * softmax_scale * log2(e) into the bf16 query rows instead and forms the weights without a running
+ * maximum; queries whose weight sum leaves 2^-100 .. 2^60 are recomputed in EXACT arithmetic inside
+ * the same launch, so results stay finite and correct for any input.  FAST perturbs a score of s
+ * nats by about 1.1e-3 * |s| nats rms (bf16 rounding of the scaled query), beside the 1.1e-3
+ * relative rms that rounding a weight to bf16 costs in both modes.
+ *   mode 0 (default): FAST iff |softmax_scale| <= INTRA_FAST_SOFTMAX_MAX_SCALE (twice 128^-1/2)
+ *   mode 1: always EXACT        mode 2: always FAST
+ * The setting is process-wide and starts from the environment variable INTRA_SOFTMAX
+ * (auto / exact / fast).  No counterpart in the reference. */
+#define INTRA_FAST_SOFTMAX_MAX_SCALE 0.1767767f
+int intra_set_softmax_mode(int mode);
+int intra_get_softmax_mode(void);
 
 /* Backward pass of intra_llm_fwd / intra_llm_fwd_ex: gradients of the inputs given the gradient
  * `dout` of the output.  The reference ships no backward kernels (README.md lists them as missing;

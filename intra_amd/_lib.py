@@ -42,6 +42,8 @@ SYMBOLS = {
     "intra_model_mask_llm_ex": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.c_void_p]),
     "intra_last_error": (ctypes.c_char_p, []),
     "intra_version": (ctypes.c_int, []),
+    "intra_set_softmax_mode": (ctypes.c_int, [ctypes.c_int]),
+    "intra_get_softmax_mode": (ctypes.c_int, []),
     "intra_plan": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.POINTER(IntraPlan)]),
     "intra_model_mask": (ctypes.c_int, [ctypes.c_int] * 7 + [ctypes.c_void_p]),
 }

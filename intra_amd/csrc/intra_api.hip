@@ -3,6 +3,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
@@ -279,9 +280,9 @@ int launch_grid(int work_items) {
   return work_items < g ? work_items : g;
 }
 
-template <class MAP, int HP, int NW>
+template <class MAP, int HP, int NW, bool FAST>
 int launch(const intra::KParams& p, int grid, hipStream_t stream) {
-  hipLaunchKernelGGL((intra::intra_fwd_kernel<MAP, HP, NW>), dim3(grid), dim3(NW * 64), 0, stream, p);
+  hipLaunchKernelGGL((intra::intra_fwd_kernel<MAP, HP, NW, FAST>), dim3(grid), dim3(NW * 64), 0, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
   return INTRA_OK;
@@ -289,21 +290,46 @@ int launch(const intra::KParams& p, int grid, hipStream_t stream) {
 
 template <class MAP>
 struct LaunchMap {
-  static int go(const intra::KParams& p, int hp, int nw, int grid, hipStream_t stream) {
+  static int go(const intra::KParams& p, int hp, int nw, bool fast, int grid, hipStream_t stream) {
     if (nw == 8) {
       switch (hp) {
-        case 4: return launch<MAP, 4, 8>(p, grid, stream);
-        case 2: return launch<MAP, 2, 8>(p, grid, stream);
-        case 1: return launch<MAP, 1, 8>(p, grid, stream);
+        case 4: return fast ? launch<MAP, 4, 8, true>(p, grid, stream) : launch<MAP, 4, 8, false>(p, grid, stream);
+        case 2: return fast ? launch<MAP, 2, 8, true>(p, grid, stream) : launch<MAP, 2, 8, false>(p, grid, stream);
+        case 1: return fast ? launch<MAP, 1, 8, true>(p, grid, stream) : launch<MAP, 1, 8, false>(p, grid, stream);
       }
     }
     return fail(INTRA_ERR_UNSUPPORTED, "no kernel for heads_per_block=%d, waves=%d", hp, nw);
   }
 };
 
+// Softmax arithmetic of the forward kernels: 0 = by softmax_scale (see use_fast_softmax), 1 = always
+// EXACT, 2 = always FAST.  Starts from the environment variable INTRA_SOFTMAX (auto / exact / fast).
+std::atomic<int>& softmax_mode() {
+  static std::atomic<int> mode{[] {
+    const char* e = getenv("INTRA_SOFTMAX");
+    if (e && !strcmp(e, "exact")) return 1;
+    if (e && !strcmp(e, "fast")) return 2;
+    return 0;
+  }()};
+  return mode;
+}
+
+// FAST rounds Q * softmax_scale * log2(e) to bf16 before the MFMA.  That perturbs a score of s nats
+// by about 2^-9 * |s| / sqrt(3) nats rms (every product q_d * k_d moves by up to 2^-9 of itself),
+// against the 2^-9 / sqrt(3) relative rms that rounding the weight to bf16 costs in either mode.
+// Up to twice the default scale d^-1/2 the scores of unit-variance inputs are a few nats and the
+// two are of one size; beyond that the fp32 scaling of the reference's arithmetic is kept.
+bool use_fast_softmax(float scale) {
+  const int mode = softmax_mode().load(std::memory_order_relaxed);
+  if (mode != 0) return mode == 2;
+  return fabsf(scale) <= INTRA_FAST_SOFTMAX_MAX_SCALE;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-// `written`: the tensor is an output, so batch entries may not alias either
+// `written`: the tensor is an output, so its elements may not alias (a zero stride over a dimension
+// larger than 1); inputs are only read, so expanded views (e.g. the gradient of a mean over tokens,
+// or one kv head broadcast over several) are fine.
 int check_strides(const char* name, const int64_t* st, int B, int S, int heads, bool written = false) {
   if (!st) return fail(INTRA_ERR_INVALID, "%s strides pointer is null", name);
   for (int i = 0; i < 3; ++i) {
@@ -312,7 +338,7 @@ int check_strides(const char* name, const int64_t* st, int B, int S, int heads, 
       return fail(INTRA_ERR_INVALID, "%s stride %d (%lld elements) breaks 16-byte alignment", name, i,
                   (long long)st[i]);
   }
-  if ((S > 1 && st[1] == 0) || (heads > 1 && st[2] == 0) || (B > 1 && st[0] == 0 && written))
+  if (written && ((S > 1 && st[1] == 0) || (heads > 1 && st[2] == 0) || (B > 1 && st[0] == 0)))
     return fail(INTRA_ERR_INVALID, "%s has a zero stride over a dimension larger than 1", name);
   return INTRA_OK;
 }
@@ -362,6 +388,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.scale_log2 = fabsf(scale) * 1.4426950408889634f;
   if (p.scale_log2 < 1e-30f) p.scale_log2 = 1e-30f;  // scale 0: uniform weights without 0 * inf on masked scores
   p.negate_q = scale < 0.f;
+  p.q_fold = scale * 1.4426950408889634f;
   p.k_rs_bytes = (uint32_t)(ks[1] * 2);
   p.v_rs_bytes = (uint32_t)(vs[1] * 2);
 
@@ -385,7 +412,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.d_nbh = make_fastdiv(B * Hkv);
   p.d_hkv = make_fastdiv(Hkv);
   p.d_hgroups = make_fastdiv(p.hgroups);
-  return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, grid, static_cast<hipStream_t>(stream));
+  return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, use_fast_softmax(scale), grid, static_cast<hipStream_t>(stream));
 }
 
 
@@ -757,7 +784,16 @@ int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint
 
 const char* intra_last_error(void) { return g_err; }
 
-int intra_version(void) { return 200; }
+int intra_version(void) { return INTRA_VERSION; }
+
+int intra_set_softmax_mode(int mode) {
+  g_err[0] = 0;
+  if (mode < 0 || mode > 2) return fail(INTRA_ERR_INVALID, "softmax mode must be 0 (auto), 1 (exact) or 2 (fast), got %d", mode);
+  softmax_mode().store(mode, std::memory_order_relaxed);
+  return INTRA_OK;
+}
+
+int intra_get_softmax_mode(void) { return softmax_mode().load(std::memory_order_relaxed); }
 
 int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
                IntraPlan* plan) {

@@ -30,6 +30,14 @@
 //  * Blocks outside a wavefront's key range are skipped; only blocks cut by a bound are masked.
 //  * The grid is persistent (about one workgroup per CU); work items are dealt per XCD so that
 //    one (batch, kv head, set) stays in one XCD's L2, in an order that balances causal triangles.
+//  * Two softmax modes.  EXACT scales the fp32 scores after the MFMA and watches every block's
+//    maximum (the reference's arithmetic, csrc/flash_attn/src/softmax.h:65-91).  FAST folds
+//    softmax_scale * log2(e) into the bf16 Q fragments once per work item and exponentiates the
+//    raw MFMA results with no running maximum at all; a query whose weight sum left the safe
+//    exponent band marks its work item in an LDS bitmap, and after the last item the workgroup
+//    runs the marked items again in EXACT mode.  The host picks FAST for |softmax_scale| up to
+//    twice the default (there the bf16 rounding of Q * c adds less noise to a weight than the
+//    bf16 rounding of the weight itself does for scores of a few nats).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -64,6 +72,7 @@ struct KParams {
   IntraGeom geom;
   float scale_log2;    // |softmax_scale| * log2(e)
   int negate_q;        // softmax_scale < 0: flip the sign of Q instead
+  float q_fold;        // FAST mode: softmax_scale * log2(e), signed, multiplied into Q
   uint32_t k_rs_bytes, v_rs_bytes;  // token strides of k and v in bytes (< 4 GiB, checked on the host)
   int n_sets;          // sets per (batch, kv head)
   int n_mblocks;       // row blocks of the largest set
@@ -86,7 +95,9 @@ constexpr int KTILE = TILE_BYTES;
 constexpr int VTILE = TILE_BYTES;
 constexpr int NKBUF = 4, NVBUF = 4;   // tiles i-1 (being overwritten) .. i+2 of K and of V
 constexpr int VBASE = NKBUF * KTILE;  // K ring then V ring
-constexpr int LDS_BYTES = NKBUF * KTILE + NVBUF * VTILE;
+constexpr int RING_BYTES = NKBUF * KTILE + NVBUF * VTILE;
+constexpr int REDO_WORDS = 64;        // bitmap of work-item rounds to run again in EXACT mode (round % 2048)
+constexpr int LDS_BYTES = RING_BYTES + REDO_WORDS * 4;
 constexpr int BLOCK32 = 8 * GROUP_STRIDE;  // 32 rows
 
 // 64 lanes x 16 bytes from per-lane global addresses to 1024 consecutive LDS bytes at lds_addr
@@ -120,13 +131,13 @@ __device__ __forceinline__ float lane_xor32_sum(float x) {
 template <int V>
 using ic = std::integral_constant<int, V>;
 
-template <class MAP, int HP, int NW>
-__global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
-  constexpr int NT = NW * 64;
+// One pass of a workgroup over its work items.  FAST: see the file comment.  REDO: visit only the
+// items whose round is marked in `redo` (the EXACT second pass of a FAST kernel).
+template <class MAP, int HP, int NW, bool FAST, bool REDO>
+__device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, uint32_t* redo) {
   constexpr int POS = NW * 32 / HP;          // in-set queries per row block
   static_assert(BN % NW == 0, "tile rows must split evenly over the wavefronts");
-
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+  static_assert(!(FAST && REDO), "the second pass is exact");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -153,6 +164,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     for (;; ++round) {
       const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
       if (slot >= p.n_slots) return false;
+      if (REDO && !((redo[(round >> 5) & (REDO_WORDS - 1)] >> (round & 31)) & 1u)) continue;
       const int pslot = (int)fd_div(slot, p.d_items_per_pair);
       const int pair = pslot * 8 + xcd;
       if (pair >= p.n_pairs) continue;
@@ -233,22 +245,25 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   };
   constexpr int PER_TILE = 2 * GROUPS_PER_WAVE;  // requests per wavefront per tile (K + V)
 
-  // K operand (A of S^T = K Q^T): lane reads 16 bytes of key row l32 at head dims 16*ks + 8*h32
-  int kaddr[8];
-#pragma unroll
-  for (int ks = 0; ks < 8; ++ks)
-    kaddr[ks] = (l32 >> 2) * GROUP_STRIDE + (l32 & 3) * 256 + (((2 * ks + h32) ^ (4 * (l32 & 3))) << 4);
-  // V^T operand (A of O^T = V^T P^T) through transposing reads.  Within each group of 16 lanes,
-  // lane i supplies the address of 4 head dims (4*(i%4)..) of key row i/4 and receives head dim i
-  // of those 4 key rows.  Lane groups 0/1 take head dims 0-15/16-31 of a 32-dim block, the upper
-  // 32 lanes the key rows 4..7 of each 8 (the next 4-row group).  vaddr[db]: 32-dim block db.
-  int vaddr[4];
+  // LDS operand addresses.  With the chunk swizzle c ^ 4i of a group, the 16-byte chunk 2*ks + h32
+  // of key row l32 (the K operand of k-step ks = 2a + b) sits at byte 64 * (a ^ r) + 32 * b +
+  // 16 * h32 of its row slot, r = l32 % 4: four lane-dependent bases (one per a) and compile-time
+  // offsets for everything else, which the ds_read offset field takes.  The bases carry the ring
+  // slot and are advanced once per tile: kb[] follows the tile AFTER the one being multiplied
+  // (whose K rows the pipeline reads ahead), vb[] the current one.
+  int kb[4], vb[4];
   {
+    const int r = l32 & 3;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) kb[a] = KTILE + (l32 >> 2) * GROUP_STRIDE + r * 256 + 64 * (a ^ r) + 16 * h32;
+    // V^T operand (A of O^T = V^T P^T) through transposing reads.  Within each group of 16 lanes,
+    // lane i supplies the address of 4 head dims (4*(i%4)..) of key row i/4 and receives head dim i
+    // of those 4 key rows.  Lane groups 0/1 take head dims 0-15/16-31 of a 32-dim block, the upper
+    // 32 lanes the key rows 4..7 of each 8 (the next 4-row group).  vb[db]: 32-dim block db.
     const int i16 = lane & 15, g2 = (lane >> 4) & 1, ri = i16 >> 2;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
-      vaddr[db] = VBASE + h32 * GROUP_STRIDE + ri * 256 + (((4 * db + 2 * g2 + ((i16 & 3) >> 1)) ^ (4 * ri)) << 4) +
-                  8 * (i16 & 1);
+      vb[db] = VBASE + h32 * GROUP_STRIDE + ri * 256 + 64 * (db ^ ri) + 16 * (2 * g2 + ((i16 & 3) >> 1)) + 8 * (i16 & 1);
   }
   // Q^T fragments: lane holds query l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
   bf16x8 qf[8];
@@ -347,10 +362,21 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
       asm volatile("" : "+v"(raw[ks]));
     }
     pair_exchange(raw);
+    if (FAST) {  // Q <- bf16(Q * softmax_scale * log2 e): the MFMA then yields exponents directly
+      const float cq = p.q_fold;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+          const uint32_t x = raw[ks][d];
+          floatx2 f = {__uint_as_float(x << 16) * cq, __uint_as_float(x & 0xffff0000u) * cq};
+          raw[ks][d] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+        }
+    }
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = __builtin_bit_cast(bf16x8, raw[ks]);
   }
-  if (p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
+  if (!FAST && p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
       qf[ks] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, qf[ks]) ^ 0x80008000u);
@@ -368,19 +394,18 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   // overflows or underflows.  fp32 and bf16 both span 2^+-126, so mref stays 0 (and costs nothing)
   // for every query whose scores stay within +-60 of it; it is re-centred on a block's maximum
   // when that maximum leaves this band upwards, or downwards before anything was accumulated.
+  // FAST mode has no reference at all (weights exp2(score), scores already in exponent units).
   float mref = 0.f;
   float l_acc[2] = {0.f, 0.f};  // two partial row sums of the weights (summed at the end)
   const float c = p.scale_log2;  // |softmax_scale| * log2(e)
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
-  // operand reads; koff / voff are byte offsets of (buffer, 32-key block) in LDS
-  auto kread = [&](int koff, int ks) { return *reinterpret_cast<const bf16x8*>(smem + koff + kaddr[ks]); };
-  auto vread = [&](int voff, int j) {  // j = 4 * t + db: keys 16t..16t+15 of the block, head dims 32db..
-    const int off = (j >> 2) * 4 * GROUP_STRIDE;
-    bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (__attribute__((address_space(3))) bf16x4*)(smem + voff + vaddr[j & 3] + off));
+  // operand reads: base register + compile-time byte offset
+  auto kread_at = [&](int base, int off) { return *reinterpret_cast<const bf16x8*>(smem + (base + off)); };
+  auto vread_at = [&](int base, int off) {
+    bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(smem + (base + off)));
     bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (__attribute__((address_space(3))) bf16x4*)(smem + voff + vaddr[j & 3] + off + 2 * GROUP_STRIDE));
+        (__attribute__((address_space(3))) bf16x4*)(smem + (base + off + 2 * GROUP_STRIDE)));
     return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
   };
 
@@ -391,11 +416,10 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     return z;
   };
   // ----- unscheduled pieces, used at the edges of a wavefront's key range
-  auto qk_block = [&](floatx16& acc, int koff) {
-    acc = zero16();
+  // K operands of a 32-key block: `delta` = its tile's ring slot minus the slot kb[] points to
+  auto load_ka = [&](bf16x8 (&ka)[8], int delta, int half) {
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kread(koff, ks), qf[ks], acc, 0, 0, 0);
+    for (int g = 0; g < 8; ++g) ka[g] = kread_at(kb[g >> 1] + delta, 32 * (g & 1) + half);
   };
   auto mask_block = [&](floatx16& s, int kb32) {
 #pragma unroll
@@ -413,8 +437,10 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     m1 = fmaxf(fmaxf(m1, s[13]), s[14]);
     return lane_xor32_max(fmaxf(fmaxf(m0, s[7]), fmaxf(m1, s[15])));
   };
-  // What can happen to a freshly computed block of raw scores q.k before it is exponentiated as
-  // exp2(score * c - mref); all of it is rare.  `mx` is the block maximum of the raw scores.
+  // EXACT mode: what can happen to a freshly computed block of raw scores q.k before it is
+  // exponentiated as exp2(score * c - mref); all of it is rare.  `mx` is the block maximum of the
+  // raw scores.  Lanes l and l + 32 hold the same query (disjoint keys, shared accumulators), so
+  // every decision here is taken per query: mx and the running sum are exchanged between the halves.
   auto settle = [&](floatx16& nxt, float mx, bool masked, int kb32) {
     if (masked) {  // block cut by a bound: mask in place, then redo the maximum
       mask_block(nxt, kb32);
@@ -422,7 +448,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     }
     const float mxs = __builtin_fmaf(mx, c, -mref);  // block maximum in exponent units
     if (__builtin_amdgcn_ballot_w64(__builtin_fabsf(mxs) > 60.f) == 0) return;  // the usual case
-    const float l_run = l_acc[0] + l_acc[1];
+    const float l_run = lane_xor32_sum(l_acc[0] + l_acc[1]);  // of the query, not of this lane's keys
     const bool need = mxs > 60.f || (l_run == 0.f && mxs < -60.f && mxs > -INFINITY);
     if (__builtin_amdgcn_ballot_w64(need) != 0) {
       const float delta = need ? mxs : 0.f;
@@ -436,6 +462,14 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
         for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
     }
   };
+  // a freshly computed block of scores, before its weights are formed
+  auto finish_scores = [&](floatx16& nxt, float mx, bool masked, int kb32) {
+    if (FAST) {
+      if (masked) mask_block(nxt, kb32);
+    } else {
+      settle(nxt, mx, masked, kb32);
+    }
+  };
 
   // ----- hand-scheduled step: QK^T of the next key block (8 MFMAs) and PV of the current one
   // (8 MFMAs) with the softmax VALU work spread between them.  One "slot" is one MFMA.  LDS
@@ -443,16 +477,24 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   // its QK^T slots, the K operands of the NEXT step's QK^T during this step's PV slots (ka lives
   // across steps and across the tile barrier: the K tile it reads was made visible by an earlier
   // barrier and is not overwritten before the next one).  The exponentials of the current block
-  // run one bf16 pair per slot in slots 0..7, the packing + row sums one slot later; the maximum
-  // of the next block is taken in the PV slots once its MFMA chain has drained.
+  // run one bf16 pair per slot in slots 0..7, the packing + row sums one slot later; in EXACT mode
+  // the maximum of the next block is taken in the PV slots once its MFMA chain has drained.
   // sched_barrier keeps the compiler from regrouping the slots.
   bf16x8 ka[8];
-  auto steady = [&](const floatx16& s, floatx16& n, int koff_next, int voff, bool mask_next, int kb32_next) {
+  // HALF: byte offset of the block's half inside its tile for the V reads (block j) and the K reads
+  // (block j + 2, one tile further): 0 or BLOCK32, the same for both.
+  auto steady = [&](const floatx16& s, floatx16& n, auto half_c, bool mask_next, int kb32_next) {
+    constexpr int HALF = decltype(half_c)::value;
     bf16x8 va[8], pb[2];
     float px[8][2];
     auto stage_e = [&](int u) {
-      px[u][0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u], c, -mref));
-      px[u][1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u + 1], c, -mref));
+      if (FAST) {
+        px[u][0] = __builtin_amdgcn_exp2f(s[2 * u]);
+        px[u][1] = __builtin_amdgcn_exp2f(s[2 * u + 1]);
+      } else {
+        px[u][0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u], c, -mref));
+        px[u][1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u + 1], c, -mref));
+      }
     };
     auto stage_c = [&](int u) {
       floatx2 f = {px[u][0], px[u][1]};
@@ -476,33 +518,35 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     };
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
-      va[g] = vread(voff, g);
+      va[g] = vread_at(vb[g & 3], (g >> 2) * 4 * GROUP_STRIDE + HALF);
       n = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[g], qf[g], g == 0 ? zero16() : n, 0, 0, 0);
       valu_slot(g);
       __builtin_amdgcn_sched_barrier(0);
     }
-    float m0, m1;
+    float m0 = 0.f, m1 = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      ka[j] = kread(koff_next, j);
+      ka[j] = kread_at(kb[j >> 1], 32 * (j & 1) + HALF);
       oacc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[j], pb[j >> 2], oacc[j & 3], 0, 0, 0);
       valu_slot(8 + j);
-      if (j == 4) m0 = fmaxf(fmaxf(n[0], n[1]), fmaxf(n[2], n[3]));
-      if (j == 5) m0 = fmaxf(fmaxf(m0, n[4]), fmaxf(n[5], fmaxf(n[6], n[7])));
-      if (j == 6) m1 = fmaxf(fmaxf(n[8], n[9]), fmaxf(n[10], n[11]));
-      if (j == 7) m1 = fmaxf(fmaxf(m1, n[12]), fmaxf(n[13], fmaxf(n[14], n[15])));
+      if (!FAST) {
+        if (j == 4) m0 = fmaxf(fmaxf(n[0], n[1]), fmaxf(n[2], n[3]));
+        if (j == 5) m0 = fmaxf(fmaxf(m0, n[4]), fmaxf(n[5], fmaxf(n[6], n[7])));
+        if (j == 6) m1 = fmaxf(fmaxf(n[8], n[9]), fmaxf(n[10], n[11]));
+        if (j == 7) m1 = fmaxf(fmaxf(m1, n[12]), fmaxf(n[13], fmaxf(n[14], n[15])));
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
-    settle(n, lane_xor32_max(fmaxf(m0, m1)), mask_next, kb32_next);
+    finish_scores(n, FAST ? 0.f : lane_xor32_max(fmaxf(m0, m1)), mask_next, kb32_next);
   };
 
-  // Step j: softmax + PV of key block j (scores in `cur`, V rows at voff) and QK^T of key block
-  // j+1 into `nxt` (its K rows at koff; those of block j+2 at koff_next).  A wavefront runs the
-  // steps jq..jp for a run of blocks jq+1..jp it looks at: in step jq only the QK^T half matters,
-  // so its scores are preset to -inf (weights 0); in step jp the QK^T half computes a block the
-  // wavefront does not look at, which the per-element mask turns into -inf.  That keeps one code
-  // path through the accumulators.  Maps with a prefix have two such runs (prefix blocks, own
-  // range); they are merged when they touch.
+  // Step j: softmax + PV of key block j (scores in `cur`, V rows in the current tile) and QK^T of
+  // key block j+1 into `nxt` (its K rows are in ka already; those of block j+2 are read meanwhile).
+  // A wavefront runs the steps jq..jp for a run of blocks jq+1..jp it looks at: in step jq only the
+  // QK^T half matters, so its scores are preset to -inf (weights 0); in step jp the QK^T half
+  // computes a block the wavefront does not look at, which the per-element mask turns into -inf.
+  // That keeps one code path through the accumulators.  Maps with a prefix have two such runs
+  // (prefix blocks, own range); they are merged when they touch.
   int jq1 = bw_lo - 1, jp1 = bw_hi, jq2 = 1, jp2 = 0;
   if (MAP::kHasPrefix && bp_hi >= 0) {
     if (bw_lo - 1 <= bp_hi) {  // the ranges touch: one run from the first prefix block on
@@ -516,18 +560,20 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     }
   }
   auto needs_mask = [&](int j) { return !block_unmasked(wb, kpre, kt_lo + 32 * j); };
-  auto step = [&](int j, floatx16& cur, floatx16& nxt, int koff, int koff_next, int voff, auto with_loader,
-                  int free_slot) {
+  // half_c: which half of its tile block j is (0 / BLOCK32).  Block j + 1 is the other half of the
+  // same tile (half 0) or the first half of the next tile (half BLOCK32).
+  auto step = [&](int j, floatx16& cur, floatx16& nxt, auto half_c, auto with_loader, int free_slot) {
+    constexpr int HALF = decltype(half_c)::value;
     if (decltype(with_loader)::value) feed_tile(free_slot);
     const bool in1 = j >= jq1 && j <= jp1, in2 = j >= jq2 && j <= jp2;
     if (!in1 && !in2) return;
     if (j == jq1 || (in2 && j == jq2)) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) cur[e] = -INFINITY;
-#pragma unroll
-      for (int g = 0; g < 8; ++g) ka[g] = kread(koff, g);
+      if (HALF == 0) load_ka(ka, k0 - k1, BLOCK32);  // second half of the current tile
+      else load_ka(ka, 0, 0);                         // first half of the next tile
     }
-    steady(cur, nxt, koff_next, voff, needs_mask(j + 1), kt_lo + 32 * (j + 1));
+    steady(cur, nxt, half_c, needs_mask(j + 1), kt_lo + 32 * (j + 1));
   };
 
   // ---------------------------------------------------------------- main loop
@@ -541,15 +587,23 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   // previous item (8 stores).  Letting PER_TILE + 8 operations pending is safe in both cases.
   tile_barrier<PER_TILE + 8>();
   if (jq1 < 0 && jp1 >= 0) {
-    qk_block(s0, k0);
-    settle(s0, block_max(s0), needs_mask(0), kt_lo);
+    load_ka(ka, k0 - k1, 0);
+    s0 = zero16();
 #pragma unroll
-    for (int g = 0; g < 8; ++g) ka[g] = kread(k0 + BLOCK32, g);
+    for (int ks = 0; ks < 8; ++ks) s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qf[ks], s0, 0, 0, 0);
+    finish_scores(s0, FAST ? 0.f : block_max(s0), needs_mask(0), kt_lo);
+    load_ka(ka, k0 - k1, BLOCK32);
   }
   for (int i = 0; i < ntiles; ++i) {
     if (i > 0) tile_barrier<PER_TILE>();
-    step(2 * i, s0, s1, k0 + BLOCK32, k1, k0, ic<1>{}, k3);
-    step(2 * i + 1, s1, s0, k1, k1 + BLOCK32, k0 + BLOCK32, ic<0>{}, 0);
+    step(2 * i, s0, s1, ic<0>{}, ic<1>{}, k3);
+    step(2 * i + 1, s1, s0, ic<BLOCK32>{}, ic<0>{}, 0);
+    const int dk = k2 - k1, dv = k1 - k0;  // +KTILE, or -3 * KTILE where the ring wraps
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      kb[a] += dk;
+      vb[a] += dv;
+    }
     const int tk = k0;
     k0 = k1; k1 = k2; k2 = k3; k3 = tk;
   }
@@ -566,6 +620,16 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   // ---------------------------------------------------------------- normalise and scatter-store
   if (wave_active) {
   const float l_tot = lane_xor32_sum(l_acc[0] + l_acc[1]);
+  if (FAST) {
+    // Weights were formed without a reference: the result is good iff the weight sum stayed inside
+    // 2^-100 .. 2^60 (no weight overflowed, and the largest ones are far from underflow).  The
+    // integer comparison of the bit patterns also catches a negative or NaN sum.
+    const uint32_t lb = __float_as_uint(l_tot);
+    const bool bad = row_valid && !(lb >= 0x0d800000u && lb <= 0x5d800000u);
+    if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0)
+      __hip_atomic_fetch_or(&redo[(cw.round >> 5) & (REDO_WORDS - 1)], 1u << (cw.round & 31), __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   if (p.lse != nullptr && row_valid && h32 == 0)  // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2
     p.lse[batch * p.lse_bs + hq * p.lse_hs + qpos * p.lse_ts] = (mref + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
@@ -604,6 +668,23 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   if (!more) break;
   cw = nw;
   }  // work items
+}
+
+template <class MAP, int HP, int NW, bool FAST>
+__global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+  uint32_t* redo = reinterpret_cast<uint32_t*>(smem + RING_BYTES);
+  if (FAST) {
+    if (threadIdx.x < REDO_WORDS) redo[threadIdx.x] = 0;  // visible after the first tile barrier
+    run_pass<MAP, HP, NW, true, false>(p, smem, redo);
+    // Every wavefront has left the first pass: its marks are in, nobody reads the ring any more and
+    // the loader's last (unused) requests have landed before new ones reuse their slots.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    const uint32_t mine = redo[threadIdx.x & (REDO_WORDS - 1)];
+    if (__builtin_amdgcn_ballot_w64(mine != 0) == 0) return;  // the usual case
+  }
+  run_pass<MAP, HP, NW, false, FAST>(p, smem, redo);
 }
 
 }  // namespace intra

@@ -1,4 +1,5 @@
-"""Python entry points of the MI355X INTRA kernels (forward only).
+"""Python entry points of the MI355X INTRA kernels: the reference's two forward calls, and a
+backward pass with autograd wrappers that the reference does not have.
 
 Same surface as the reference's intra_attn/interface.py:12-66: `intra_llm_attn` and
 `intra_image_attn` take q, k, v of shape (batch, seqlen, heads, 128) in bfloat16 on the GPU and
@@ -27,12 +28,29 @@ def _aligned(x):
     return x.stride(-1) == 1 and x.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in x.stride()[:-1])
 
 
-def _check(q, k, v):
+SOFTMAX_MODES = {"auto": 0, "exact": 1, "fast": 2}
+
+
+def set_softmax_mode(mode):
+    """Softmax arithmetic of the forward kernels, process-wide: "exact" scales the fp32 scores after
+    the first product like the reference (csrc/flash_attn/src/softmax.h:65-91); "fast" folds the
+    scale into the bf16 queries and recomputes, exactly, the queries whose weight sum leaves the
+    safe exponent range; "auto" (default) picks fast up to twice the default softmax_scale."""
+    if _C.intra_set_softmax_mode(SOFTMAX_MODES[mode]) != _lib.INTRA_OK:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
+
+
+def get_softmax_mode():
+    return {v: k for k, v in SOFTMAX_MODES.items()}[_C.intra_get_softmax_mode()]
+
+
+def _check(q, k, v, forward_call=True):
     # reference: intra_attn/interface.py:17-23 (same conditions, same exception types and texts)
     for x in (q, k, v):
         if not x.is_cuda or x.dtype != torch.bfloat16 or x.shape[-1] != 128:
             raise ValueError("INTRA kernels need CUDA bfloat16 tensors with head_dim 128")
-    if torch.is_grad_enabled() and any(x.requires_grad for x in (q, k, v)):
+    # the plain forward calls record no graph (intra_llm_attn_func / intra_image_attn_func do)
+    if forward_call and torch.is_grad_enabled() and any(x.requires_grad for x in (q, k, v)):
         raise RuntimeError("INTRA kernels are forward-only; call them under torch.no_grad()")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise ValueError("q, k, v must be (batch, seqlen, heads, 128)")
@@ -133,7 +151,7 @@ def intra_llm_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", group_num=8, 
     of the forward call.  block_scatter with offset != 0 needs block % 256 == 0.  The reference has
     no backward kernels (its training runs differentiate masked SDPA,
     experiments/llm/llama_intra.py:26)."""
-    q, k, v = _check(q, k, v)
+    q, k, v = _check(q, k, v, forward_call=False)
     ids = dict(LLM_PATTERNS, **EXTRA_LLM_PATTERNS)
     if pattern not in ids:
         raise ValueError(f"unknown pattern {pattern!r}")
@@ -195,7 +213,7 @@ def intra_image_attn_bwd(q, k, v, out, lse, dout, pattern="scatter", width=64, s
     """Gradients (dq, dk, dv) of intra_image_attn, given the forward results `out`, `lse`
     (return_lse=True) and the gradient `dout` of `out`.  The reference has no backward kernels (its
     FLUX training differentiates masked SDPA, experiments/flux/intra_processor.py:138-142)."""
-    q, k, v = _check(q, k, v)
+    q, k, v = _check(q, k, v, forward_call=False)
     if width not in (64, 128):
         raise ValueError("image kernels are compiled for width 64 and 128")
     if q.shape[1] != TEXT_LEN + width * width:

@@ -103,6 +103,37 @@ def test_fwd_validates_before_touching_the_gpu(lib):
     assert "expected 512 text" in _lib.last_error()
 
 
+def test_zero_strides_are_for_inputs_only(lib):
+    # expanded (stride 0) views are fine where the kernels only read; outputs may not alias
+    st = (ctypes.c_int64 * 3)(128 * 4 * 128, 4 * 128, 128)
+    tok0 = (ctypes.c_int64 * 3)(128 * 4 * 128, 0, 128)
+    head0 = (ctypes.c_int64 * 3)(128 * 4 * 128, 4 * 128, 0)
+    ptr = 1 << 20  # never dereferenced: the NaN scale fails validation after the stride checks
+    nan = float("nan")
+    for inputs in ((tok0, st, st), (st, head0, st), (st, st, head0), (tok0, tok0, tok0)):
+        assert lib.intra_llm_fwd(ptr, ptr, ptr, ptr, 1, 128, 4, 4, *inputs, st, 0, 8, 576, nan, None) == 1
+        assert "finite" in _lib.last_error()
+    for out in (tok0, head0):
+        assert lib.intra_llm_fwd(ptr, ptr, ptr, ptr, 1, 128, 4, 4, st, st, st, out, 0, 8, 576, nan, None) == 1
+        assert "o has a zero stride" in _lib.last_error()
+
+
+def test_version_and_softmax_mode(lib):
+    import intra_amd
+    major, minor, patch = (int(x) for x in intra_amd.__version__.split("."))
+    assert lib.intra_version() == major * 10000 + minor * 100 + patch
+    start = lib.intra_get_softmax_mode()
+    try:
+        for mode in (1, 2, 0):
+            assert lib.intra_set_softmax_mode(mode) == 0 and lib.intra_get_softmax_mode() == mode
+        assert lib.intra_set_softmax_mode(3) == 1 and "softmax mode" in _lib.last_error()
+        assert lib.intra_get_softmax_mode() == 0
+        intra_amd.set_softmax_mode("exact")
+        assert intra_amd.get_softmax_mode() == "exact"
+    finally:
+        lib.intra_set_softmax_mode(start)
+
+
 def test_lse_entry_points_validate_their_extra_arguments(lib):
     st = (ctypes.c_int64 * 3)(128 * 4 * 128, 4 * 128, 128)
     ls = (ctypes.c_int64 * 3)(4 * 128, 128, 1)

@@ -7,6 +7,7 @@ test uses 2e-2 and reports ~1e-3 observed)."""
 import pytest
 import torch
 
+import intra_amd
 import oracle
 from intra_amd import intra_image_attn, intra_llm_attn
 
@@ -229,7 +230,11 @@ def test_oracle_on_gpu_equals_oracle_on_cpu():
 
 # fp32 log-sum-exp.  The kernel sums the bf16-rounded weights (the ones PV multiplies), each off by
 # at most 2^-8 relative, so the sum is too and the logarithm by at most ln(1 + 2^-8) = 3.9e-3.
-LSE_ATOL = 5e-3
+# With the scale folded into bf16 Q (the FAST arithmetic that the default scale gets) the scores
+# themselves move by up to 2^-9 * |scale| * sum_d |q_d k_d| (rms about 1.1e-3 of the score in nats),
+# and lse follows the largest scores: 1e-2 covers N(0,1) inputs at these scales.
+LSE_ATOL_EXACT = 5e-3
+LSE_ATOL = 1e-2
 
 
 @pytest.mark.parametrize("kind,fn,S,H,Hkv,kw", [
@@ -240,17 +245,22 @@ LSE_ATOL = 5e-3
     ("image/gather0", intra_image_attn, 4608, 4, 2, dict(width=64)),
 ])
 @pytest.mark.parametrize("scale", [None, -0.07])
-def test_lse_output(kind, fn, S, H, Hkv, kw, scale):
+@pytest.mark.parametrize("mode", ["exact", "auto"])
+def test_lse_output(kind, fn, S, H, Hkv, kw, scale, mode):
     q, k, v = make_qkv(2, S, H, Hkv, seed=21)
-    with torch.no_grad():
-        out, lse = fn(q, k, v, kind.split("/")[1], softmax_scale=scale, return_lse=True, **kw)
-        plain = fn(q, k, v, kind.split("/")[1], softmax_scale=scale, **kw)
+    intra_amd.set_softmax_mode(mode)
+    try:
+        with torch.no_grad():
+            out, lse = fn(q, k, v, kind.split("/")[1], softmax_scale=scale, return_lse=True, **kw)
+            plain = fn(q, k, v, kind.split("/")[1], softmax_scale=scale, **kw)
+    finally:
+        intra_amd.set_softmax_mode("auto")
     assert torch.equal(out, plain)
     assert lse.shape == (2, H, S) and lse.dtype == torch.float32
     mask = oracle.mask_rows(kind, S, device=DEV, **kw)
     ref = oracle.masked_lse_rows(q, k, mask, softmax_scale=scale)
     err = (lse - ref).abs().max().item()
-    assert err <= LSE_ATOL, f"{kind}: lse max|err|={err:.3e}"
+    assert err <= (LSE_ATOL_EXACT if mode == "exact" else LSE_ATOL), f"{kind}: lse max|err|={err:.3e}"
 
 
 def test_lse_depends_on_q_and_k_only():
@@ -375,7 +385,8 @@ def test_random_llm_shapes(case):
         out, lse = intra_llm_attn(q, k, v, kind, softmax_scale=scale, return_lse=True, **kw)
     check(out, q, k, v, f"llm/{kind}", scale=scale, rtol=2.0 ** -7, **kw)
     ref = oracle.masked_lse_rows(q, k, oracle.mask_rows(f"llm/{kind}", S, device=DEV, **kw), softmax_scale=scale)
-    assert (lse - ref).abs().max().item() <= LSE_ATOL
+    # random scales up to twice the default: the score noise of the folded scale grows with the scores
+    assert bool(((lse - ref).abs() <= LSE_ATOL + 2e-3 * ref.abs()).all())
 
 
 @pytest.mark.parametrize("width,text_len,H,Hkv", [(24, 72, 4, 4), (40, 8, 8, 2), (16, 200, 2, 1), (32, 96, 4, 1)])
