@@ -209,6 +209,28 @@ int intra_model_mask_llm_bwd(int pattern, int S, int group_num, int window, int 
                              int n_sink, uint8_t* count);
 int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint8_t* count);
 
+/* ------------------------------------------------------------------ measurement aids
+ * None of these has a counterpart in the reference; they exist so that the numbers quoted for the
+ * kernels can be reproduced from this library.
+ *
+ * intra_diag_set_buffer: libraries built with -DINTRA_DIAG_TIMERS (python -m intra_amd.build --diag
+ * makes intra_amd/libintra_hip_diag.so) time the phases of a work item inside the forward kernel.
+ * `counters` is device memory for 8 int64 values per workgroup of the largest launch to come,
+ * zeroed by the caller; every forward launch whose grid fits ADDS per workgroup: 100 MHz wall-clock
+ * ticks of [0] item set-up, [1] the first barrier, [2] the first key block, [3] the tile loop,
+ * [4] look-up of the next item, its Q request, normalisation and stores; [5] work items, [6] key
+ * tiles, [7] shader cycles of the tile loops.  NULL switches it off.  A production build returns
+ * INTRA_ERR_UNSUPPORTED and never touches such a buffer.
+ *
+ * intra_diag_mfma_ceiling: one launch of `workgroups` x 8 wavefronts that issue nothing but
+ * v_mfma_f32_32x32x16_bf16 (16 per iteration and wavefront, four independent accumulators) on
+ * operands read once from `table` (131072 bytes the caller fills: constant or random bf16 bits).
+ * `sink` takes workgroups * 512 floats, `clocks` per workgroup {shader cycles, 100 MHz ticks} of
+ * the loop.  Work per launch: workgroups * 8 * iters * 16 * 32768 flop.  Allocates nothing. */
+int intra_diag_set_buffer(long long* counters, int64_t n_values);
+int intra_diag_mfma_ceiling(const void* table, float* sink, long long* clocks, int workgroups,
+                            int iters, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -6,6 +6,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 # INTRA_HIP_LIB overrides the in-tree build (e.g. to try another build of the same ABI)
 LIB_PATH = os.environ.get("INTRA_HIP_LIB") or os.path.join(_HERE, "libintra_hip.so")
+DIAG_LIB_PATH = os.path.join(_HERE, "libintra_hip_diag.so")  # the -DINTRA_DIAG_TIMERS build (measurement only)
 
 INTRA_OK, INTRA_ERR_INVALID, INTRA_ERR_UNSUPPORTED, INTRA_ERR_HIP = 0, 1, 2, 3
 
@@ -44,6 +45,8 @@ SYMBOLS = {
     "intra_version": (ctypes.c_int, []),
     "intra_set_softmax_mode": (ctypes.c_int, [ctypes.c_int]),
     "intra_get_softmax_mode": (ctypes.c_int, []),
+    "intra_diag_set_buffer": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64]),
+    "intra_diag_mfma_ceiling": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int, ctypes.c_int, ctypes.c_void_p]),
     "intra_plan": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.POINTER(IntraPlan)]),
     "intra_model_mask": (ctypes.c_int, [ctypes.c_int] * 7 + [ctypes.c_void_p]),
 }

@@ -1,6 +1,7 @@
 """Builds libintra_hip.so for gfx950 with hipcc (no torch or CUDA-compat headers involved).
 
-    python -m intra_amd.build
+    python -m intra_amd.build            # intra_amd/libintra_hip.so
+    python -m intra_amd.build --diag     # intra_amd/libintra_hip_diag.so, with in-kernel phase timers
 
 Takes the place of the reference's CUDAExtension build (setup.py:28-68).
 """
@@ -29,9 +30,16 @@ def hipcc_path():
     raise RuntimeError("hipcc not found; set HIPCC or install ROCm")
 
 
-def build(verbose=False, extra_flags=()):
-    """Compile the library in-tree and return its path."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, SRC, "-o", LIB + ".tmp"]
+DIAG_LIB = os.path.join(HERE, "libintra_hip_diag.so")
+
+
+def build(verbose=False, extra_flags=(), diag=False):
+    """Compile the library in-tree and return its path.  diag=True builds the measurement variant
+    libintra_hip_diag.so (same sources with the in-kernel phase timers compiled in) instead."""
+    lib = DIAG_LIB if diag else LIB
+    if diag:
+        extra_flags = ("-DINTRA_DIAG_TIMERS", *extra_flags)
+    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, SRC, "-o", lib + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -40,9 +48,10 @@ def build(verbose=False, extra_flags=()):
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
     if verbose and out.strip():
         print(out)
-    os.replace(LIB + ".tmp", LIB)
-    return LIB
+    os.replace(lib + ".tmp", lib)
+    return lib
 
 
 if __name__ == "__main__":
-    print(build(verbose=True, extra_flags=sys.argv[1:]))
+    args = sys.argv[1:]
+    print(build(verbose=True, extra_flags=[a for a in args if a != "--diag"], diag="--diag" in args))

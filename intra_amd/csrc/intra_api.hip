@@ -13,6 +13,7 @@
 #include "../../include/intra_hip.h"
 #include "intra_kernel.hip.h"
 #include "intra_bwd_kernel.hip.h"
+#include "intra_diag.hip.h"
 
 namespace {
 
@@ -302,6 +303,10 @@ struct LaunchMap {
   }
 };
 
+// Device buffer of the phase timers of an INTRA_DIAG_TIMERS build (intra_diag_set_buffer)
+std::atomic<long long*> g_diag{nullptr};
+std::atomic<int64_t> g_diag_values{0};
+
 // Softmax arithmetic of the forward kernels: 0 = by softmax_scale (see use_fast_softmax), 1 = always
 // EXACT, 2 = always FAST.  Starts from the environment variable INTRA_SOFTMAX (auto / exact / fast).
 std::atomic<int>& softmax_mode() {
@@ -412,6 +417,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.d_nbh = make_fastdiv(B * Hkv);
   p.d_hkv = make_fastdiv(Hkv);
   p.d_hgroups = make_fastdiv(p.hgroups);
+  p.diag = (int64_t)grid * intra::DIAG_SLOTS <= g_diag_values.load() ? g_diag.load() : nullptr;
   return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, use_fast_softmax(scale), grid, static_cast<hipStream_t>(stream));
 }
 
@@ -794,6 +800,36 @@ int intra_set_softmax_mode(int mode) {
 }
 
 int intra_get_softmax_mode(void) { return softmax_mode().load(std::memory_order_relaxed); }
+
+int intra_diag_set_buffer(long long* counters, int64_t n_values) {
+  g_err[0] = 0;
+#ifdef INTRA_DIAG_TIMERS
+  if (counters != nullptr && (n_values < intra::DIAG_SLOTS || (reinterpret_cast<uintptr_t>(counters) & 7)))
+    return fail(INTRA_ERR_INVALID, "the timer buffer must be 8-byte aligned and hold at least %d values", intra::DIAG_SLOTS);
+  g_diag_values.store(0);
+  g_diag.store(counters);
+  g_diag_values.store(counters ? n_values : 0);
+  return INTRA_OK;
+#else
+  (void)counters;
+  (void)n_values;
+  return fail(INTRA_ERR_UNSUPPORTED, "this library was built without -DINTRA_DIAG_TIMERS (python -m intra_amd.build --diag)");
+#endif
+}
+
+int intra_diag_mfma_ceiling(const void* table, float* sink, long long* clocks, int workgroups, int iters,
+                            void* hip_stream) {
+  g_err[0] = 0;
+  if (!table || !sink || !clocks) return fail(INTRA_ERR_INVALID, "table, sink and clocks must be non-null device pointers");
+  if (!aligned16(table)) return fail(INTRA_ERR_INVALID, "table must be 16-byte aligned");
+  if (workgroups < 1 || workgroups > 65536 || iters < 1)
+    return fail(INTRA_ERR_INVALID, "workgroups must be in [1, 65536] and iters positive (got %d, %d)", workgroups, iters);
+  hipLaunchKernelGGL(intra::mfma_ceiling_kernel, dim3(workgroups), dim3(512), 0, static_cast<hipStream_t>(hip_stream),
+                     static_cast<const uint4*>(table), sink, iters, clocks);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+  return INTRA_OK;
+}
 
 int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
                IntraPlan* plan) {

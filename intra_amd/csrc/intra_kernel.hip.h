@@ -81,7 +81,20 @@ struct KParams {
   int items_per_pair;  // hgroups * n_mblocks
   int n_slots;         // work items per XCD: ceil(n_pairs / 8) * items_per_pair
   FastDiv d_items_per_pair, d_nbh, d_hkv, d_hgroups;  // divisions by items_per_pair, B * Hkv, Hkv, hgroups
+  long long* diag;     // INTRA_DIAG_TIMERS builds: DIAG_SLOTS counters per workgroup, or null
 };
+
+// Phase timers of diagnostic builds (-DINTRA_DIAG_TIMERS): wavefront 0 of every workgroup adds up,
+// over its work items, the 100 MHz wall clock spent in each phase and the shader cycles of the tile
+// loop, and stores DIAG_SLOTS values at the end: [0] item set-up, [1] first barrier, [2] first key
+// block, [3] tile loop, [4] next-item look-up, Q request, normalisation and stores, [5] work items,
+// [6] tiles, [7] shader cycles of the tile loops.  Production builds compile none of it.
+constexpr int DIAG_SLOTS = 8;
+#ifdef INTRA_DIAG_TIMERS
+#define INTRA_DIAG(...) __VA_ARGS__
+#else
+#define INTRA_DIAG(...)
+#endif
 
 constexpr int BN = 64;             // keys per tile (one barrier per tile)
 // LDS tile layout.  A tile is 16 groups of 4 rows; a group is 1024 contiguous bytes (what one
@@ -226,6 +239,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   };
   Where cw;
   if (!locate(0, cw)) return;
+  INTRA_DIAG(long long dg[DIAG_SLOTS] = {0, 0, 0, 0, 0, 0, 0, 0};)
   Feed fd = feed_for(cw, -1);
   auto feed_tile = [&](int slot_off) {  // request the next K and V tile of the stream into a ring slot
 #pragma unroll
@@ -309,6 +323,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   load_q(cw);  // after the tile requests: the load counter is in order, so Q arrives last
 
   for (;;) {
+  INTRA_DIAG(const long long t_a = wall_clock64();)
   const int set = cw.set, batch = cw.batch, kvh = cw.kvh, mblk = cw.mblk, hg = cw.hg;
   const int t0 = mblk * POS;
   const MAP map(p.geom, set, t0);
@@ -585,7 +600,9 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   // At the start of a work item a wavefront has issued, after the requests for tiles 0 and 1:
   // those for tile 2, its own Q (8 loads) and, unless it was idle, the output rows of the
   // previous item (8 stores).  Letting PER_TILE + 8 operations pending is safe in both cases.
+  INTRA_DIAG(const long long t_b = wall_clock64();)
   tile_barrier<PER_TILE + 8>();
+  INTRA_DIAG(const long long t_c = wall_clock64();)
   if (jq1 < 0 && jp1 >= 0) {
     load_ka(ka, k0 - k1, 0);
     s0 = zero16();
@@ -594,6 +611,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     finish_scores(s0, FAST ? 0.f : block_max(s0), needs_mask(0), kt_lo);
     load_ka(ka, k0 - k1, BLOCK32);
   }
+  INTRA_DIAG(const long long t_d = wall_clock64(); const long long c_d = __builtin_readcyclecounter();)
   for (int i = 0; i < ntiles; ++i) {
     if (i > 0) tile_barrier<PER_TILE>();
     step(2 * i, s0, s1, ic<0>{}, ic<1>{}, k3);
@@ -608,6 +626,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     k0 = k1; k1 = k2; k2 = k3; k3 = tk;
   }
 
+  INTRA_DIAG(const long long t_e = wall_clock64(); dg[7] += __builtin_readcyclecounter() - c_d;)
   // Q of the next work item is requested before the output rows of this one are stored, so that
   // it travels while the epilogue runs (qf is dead here).
   // The loader is ahead by three tiles, so it usually knows the next work item already.
@@ -665,9 +684,13 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
       *reinterpret_cast<u32x4*>(((i & 1) ? orow_b : orow_a) + 32 * (i >> 1)) = pk[i];
   }
   }
+  INTRA_DIAG(dg[0] += t_b - t_a; dg[1] += t_c - t_b; dg[2] += t_d - t_c; dg[3] += t_e - t_d;
+             dg[4] += wall_clock64() - t_e; dg[5] += 1; dg[6] += ntiles;)
   if (!more) break;
   cw = nw;
   }  // work items
+  INTRA_DIAG(if (p.diag != nullptr && tid == 0) for (int i = 0; i < DIAG_SLOTS; ++i)
+               p.diag[(size_t)blockIdx.x * DIAG_SLOTS + i] += dg[i];)
 }
 
 template <class MAP, int HP, int NW, bool FAST>
