@@ -1,20 +1,34 @@
-"""Per-pattern latency table of the INTRA kernels on MI355X.
+"""Per-pattern latency table of the INTRA kernels on MI355X, and two measurement modes.
 
-Same protocol and CLI as the reference's benchmarks/bench_kernel.py:23-34,91-111 (median of
---iters event-timed calls after --warmup calls; `llm` and `image` modes), with the rows extended
-by effective TFLOP/s (unmasked pairs only) and the fraction of the bf16 dense MFMA peak.  The rows
-keep the reference's keys with the latency in ms as value (benchmarks/results/*.json); the
-additions are `<key>_tflops`, `<key>_pct_peak` and the `*_run` stacks.
+`llm` and `image`: protocol and CLI of the reference's benchmarks/bench_kernel.py:23-34,91-111
+(median of --iters event-timed calls after --warmup calls), rows with the reference's keys and the
+latency in ms as value (benchmarks/results/*.json), extended by `<key>_tflops` (unmasked pairs
+only), `<key>_pct_peak` (of the bf16 dense MFMA peak), the `*_run` stacks and, with --cpu, the
+dense-mask specification timed on the host cores (`<key>_cpu_ms`, `cpu_cores`).
 
     python -m intra_amd.bench_kernel llm   --seqlens 4096,8192,16384,32768,65536
     python -m intra_amd.bench_kernel image
+
+`phases`: where a workgroup's time goes, from timers inside the kernel.  Needs the measurement
+build of the library (python -m intra_amd.build --diag), selected through INTRA_HIP_LIB:
+
+    INTRA_HIP_LIB=intra_amd/libintra_hip_diag.so python -m intra_amd.bench_kernel phases \
+        --pattern scatter --seqlen 32768 [--softmax exact]
+
+`ceiling`: what the matrix cores sustain with nothing else running, with constant and with random
+operand bits, and the clock they run at (the board is power-limited):
+
+    python -m intra_amd.bench_kernel ceiling
 """
 import argparse
+import ctypes
 import json
+import time
 
 import torch
 import torch.nn.functional as F
 
+import intra_amd
 from intra_amd import _lib, intra_image_attn, intra_image_attn_bwd, intra_llm_attn, intra_llm_attn_bwd
 from intra_amd.interface import TEXT_LEN
 
@@ -22,21 +36,37 @@ PEAK_BF16_TFLOPS = 2516.6
 
 
 def median_ms(fn, warmup, iters):
+    """Median latency of fn() in ms.  After `warmup` untimed calls, each of `iters` calls sits
+    between two events on the current stream and has finished before the next one is issued."""
     for _ in range(warmup):
         fn()
-    times = []
-    for _ in range(iters):
-        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        start.record()
+    samples = []
+    while len(samples) < iters:
+        tic, toc = (torch.cuda.Event(enable_timing=True) for _ in range(2))
+        tic.record()
         fn()
-        end.record()
-        torch.cuda.synchronize()
-        times.append(start.elapsed_time(end))
-    return sorted(times)[len(times) // 2]
+        toc.record()
+        toc.synchronize()
+        samples.append(tic.elapsed_time(toc))
+    samples.sort()
+    return samples[iters // 2]
+
+
+def cpu_spec_ms(q, k, v, mask_fn):
+    """The dense-mask specification (masked fp32 attention over an S x S boolean mask, what the
+    reference's intra_attn/reference.py:78-83 defines) on the host cores: one warm-up, median of 3."""
+    from intra_attn.reference import masked_attention
+    qc, kc, vc = (x.cpu() for x in (q, k, v))
+    mask = mask_fn()
+    times = []
+    for _ in range(4):
+        t0 = time.perf_counter()
+        masked_attention(qc, kc, vc, mask)
+        times.append((time.perf_counter() - t0) * 1e3)
+    return round(sorted(times[1:])[1], 2)
 
 
 def pairs(domain, pattern, B, S, H, Hkv, a0, a1):
-    import ctypes
     plan = _lib.IntraPlan()
     rc = _lib.load().intra_plan(domain, pattern, B, S, H, Hkv, a0, a1, ctypes.byref(plan))
     assert rc == 0, _lib.last_error()
@@ -44,7 +74,6 @@ def pairs(domain, pattern, B, S, H, Hkv, a0, a1):
 
 
 def pairs_ex(pattern, B, S, H, Hkv, group_num, window, block, offset, n_sink):
-    import ctypes
     plan = _lib.IntraPlan()
     rc = _lib.load().intra_plan_llm_ex(pattern, B, S, H, Hkv, group_num, window, block, offset, n_sink,
                                        ctypes.byref(plan))
@@ -82,26 +111,24 @@ def bench_llm(args):
         if args.dense:
             ms = median_ms(lambda: dense_sdpa(q, k, v, True), args.warmup, args.iters)
             put(r, "dense", ms, S * (S + 1) // 2, B, H)
-        if args.cpu and S <= 8192:
-            # torch SDPA on the host cores for the dense causal problem, fp32: the scale of a CPU run
-            # beside the GPU rows (one warm-up, median of 3)
-            import time
-            qc, kc, vc = (x.float().cpu() for x in (q, k, v))
-            times = []
-            for _ in range(4):
-                t0 = time.perf_counter()
-                dense_sdpa(qc, kc, vc, True)
-                times.append((time.perf_counter() - t0) * 1e3)
-            r["dense_cpu_ms"] = round(sorted(times[1:])[1], 2)
+        cpu = args.cpu and S <= 8192
+        if cpu:
+            from intra_attn import reference as spec
             r["cpu_cores"] = torch.get_num_threads()
         for G in args.groups:
             ms = median_ms(lambda: intra_llm_attn(q, k, v, "scatter", group_num=G), args.warmup, args.iters)
             put(r, f"scatter_g{G}", ms, pairs(0, 0, B, S, H, Hkv, G, 576), B, H)
+            if cpu:
+                r[f"scatter_g{G}_cpu_ms"] = cpu_spec_ms(q, k, v, lambda: spec.llm_scatter_mask(S, G))
         if S % 64 == 0:
             ms = median_ms(lambda: intra_llm_attn(q, k, v, "gather1", group_num=8), args.warmup, args.iters)
             put(r, "gather1_g8", ms, pairs(0, 1, B, S, H, Hkv, 8, 576), B, H)
+            if cpu:
+                r["gather1_g8_cpu_ms"] = cpu_spec_ms(q, k, v, lambda: spec.llm_gather1_mask(S, 8))
         ms = median_ms(lambda: intra_llm_attn(q, k, v, "window", window=576), args.warmup, args.iters)
         put(r, "window576", ms, pairs(0, 4, B, S, H, Hkv, 8, 576), B, H)
+        if cpu:
+            r["window576_cpu_ms"] = cpu_spec_ms(q, k, v, lambda: spec.llm_window_mask(S, 576))
         if "scatter_g2" in r:
             # the reference's arithmetic for the 32-layer g2s4 schedule (bench_kernel.py:66-68) ...
             r["g2s4_32layer"] = round(4 * r["scatter_g2"] + 28 * r["window576"], 3)
@@ -192,6 +219,11 @@ def bench_image(args):
         for pattern, pid in (("scatter", 0), ("gather0", 4)):
             ms = median_ms(lambda: intra_image_attn(q, k, v, pattern, width), args.warmup, args.iters)
             put(r, pattern, ms, pairs(1, pid, B, S, H, H, width, TEXT_LEN), B, H)
+            if args.cpu and S <= 8192:
+                from intra_attn import reference as spec
+                mask_fn = spec.image_scatter_mask if pattern == "scatter" else spec.image_gather0_mask
+                r[pattern + "_cpu_ms"] = cpu_spec_ms(q, k, v, lambda: mask_fn(width))
+                r["cpu_cores"] = torch.get_num_threads()
         r["interleaved_mean"] = round((r["scatter"] + r["gather0"]) / 2, 4)  # layers alternate the two patterns
         if args.backward:
             dout = qkv(B, S, H, H, seed=1)[0]
@@ -207,9 +239,91 @@ def bench_image(args):
     return rows
 
 
+PHASES = ["item set-up", "first barrier", "first key block", "tile loop", "next item, Q request, normalise, store"]
+
+
+@torch.no_grad()
+def bench_phases(args):
+    """Sum over a launch of the in-kernel phase timers (see include/intra_hip.h, intra_diag_set_buffer)."""
+    lib = _lib.load()
+    n_wg = 4096
+    buf = torch.zeros(n_wg * 8, dtype=torch.int64, device="cuda")
+    if lib.intra_diag_set_buffer(buf.data_ptr(), buf.numel()) != 0:
+        raise SystemExit(f"{_lib.last_error()}; run with INTRA_HIP_LIB={_lib.DIAG_LIB_PATH}")
+    intra_amd.set_softmax_mode(args.softmax)
+    S = TEXT_LEN + args.width ** 2 if args.pattern.startswith("image") else args.seqlen
+    if args.pattern.startswith("image"):
+        q, k, v = qkv(args.batch, S, args.image_heads, args.image_heads)
+        call = lambda: intra_image_attn(q, k, v, args.pattern.split("_")[1], args.width)
+    else:
+        q, k, v = qkv(args.batch, S, args.heads, args.kv_heads)
+        kw = {"scatter": dict(group_num=args.groups[-1]), "gather1": dict(group_num=8), "window": dict(window=576)}[args.pattern]
+        call = lambda: intra_llm_attn(q, k, v, args.pattern, **kw)
+    for _ in range(args.warmup):
+        call()
+    torch.cuda.synchronize()
+    buf.zero_()
+    for _ in range(args.iters):
+        call()
+    torch.cuda.synchronize()
+    lib.intra_diag_set_buffer(None, 0)
+    d = buf.view(-1, 8).double().cpu()
+    d = d[d[:, 5] > 0] / args.iters
+    items, tiles = d[:, 5].mean().item(), d[:, 6].mean().item()
+    res = {"pattern": args.pattern, "seqlen": S, "softmax": args.softmax, "workgroups": d.shape[0],
+           "items_per_workgroup": round(items, 2), "tiles_per_item": round(tiles / items, 2), "us_per_item": {}}
+    for i, name in enumerate(PHASES):
+        res["us_per_item"][name] = round(d[:, i].mean().item() / 100 / items, 3)  # 100 MHz ticks
+    loop_us = d[:, 3].mean().item() / 100
+    res["us_per_tile"] = round(loop_us / tiles, 4)
+    res["cycles_per_tile"] = round(d[:, 7].mean().item() / tiles, 1)
+    res["shader_clock_mhz"] = round(d[:, 7].mean().item() / loop_us, 1)
+    res["us_per_workgroup"] = {"mean": round(d[:, :5].sum(1).mean().item() / 100, 1),
+                               "max": round(d[:, :5].sum(1).max().item() / 100, 1)}
+    res["share_outside_tile_loop"] = round(1 - d[:, 3].sum().item() / d[:, :5].sum().item(), 4)
+    print(json.dumps(res), flush=True)
+    return [res]
+
+
+def bench_ceiling(args):
+    """MFMA-only launch (8 wavefronts per CU on every CU, nothing but v_mfma_f32_32x32x16_bf16) with
+    constant and with random operand bits: TFLOP/s and the shader clock it ran at."""
+    lib = _lib.load()
+    n_wg = torch.cuda.get_device_properties(0).multi_processor_count
+    iters = 20000
+    sink = torch.empty(n_wg * 512, dtype=torch.float32, device="cuda")
+    clocks = torch.zeros(n_wg * 2, dtype=torch.int64, device="cuda")
+    g = torch.Generator().manual_seed(1)
+    tables = {"constant 1.0": torch.full((65536,), 1.0).to(torch.bfloat16),
+              "random N(0,1)": torch.randn(65536, generator=g).to(torch.bfloat16)}
+    rows = []
+    for name, host in tables.items():
+        table = host.cuda()
+        stream = torch.cuda.current_stream().cuda_stream
+        best = None
+        for rep in range(4):
+            tic, toc = (torch.cuda.Event(enable_timing=True) for _ in range(2))
+            tic.record()
+            rc = lib.intra_diag_mfma_ceiling(table.data_ptr(), sink.data_ptr(), clocks.data_ptr(), n_wg, iters, stream)
+            assert rc == 0, _lib.last_error()
+            toc.record()
+            toc.synchronize()
+            ms = tic.elapsed_time(toc)
+            c = clocks.view(-1, 2).double().cpu()
+            row = {"operands": name, "workgroups": n_wg, "ms": round(ms, 3),
+                   "tflops": round(n_wg * 8 * iters * 16 * 32768 / (ms * 1e-3) / 1e12, 1),
+                   "shader_clock_mhz": round((c[:, 0] / c[:, 1]).mean().item() * 100, 1)}
+            if rep > 0 and (best is None or row["ms"] < best["ms"]):  # first launch: clock still ramping
+                best = row
+        best["pct_peak"] = round(100 * best["tflops"] / PEAK_BF16_TFLOPS, 1)
+        rows.append(best)
+        print(json.dumps(best), flush=True)
+    return rows
+
+
 def main():
     p = argparse.ArgumentParser()
-    p.add_argument("mode", choices=["llm", "image"])
+    p.add_argument("mode", choices=["llm", "image", "phases", "ceiling"])
     p.add_argument("--seqlens", default="4096,8192,16384,32768,65536")
     p.add_argument("--groups", default="2,8")
     p.add_argument("--batch", type=int, default=1)
@@ -219,18 +333,25 @@ def main():
     p.add_argument("--widths", default="64,128", help="image: latent grid sides (64: 1024 x 1024, 128: 2048 x 2048)")
     p.add_argument("--warmup", type=int, default=10)
     p.add_argument("--iters", type=int, default=50)
-    p.add_argument("--dense", action="store_true", help="also time torch SDPA on the dense problem")
-    p.add_argument("--cpu", action="store_true", help="llm: also time dense causal SDPA on the host CPU (S <= 8192)")
+    p.add_argument("--no-dense", dest="dense", action="store_false",
+                   help="skip torch SDPA on the dense problem (the reference's `dense` column)")
+    p.add_argument("--cpu", action="store_true",
+                   help="also time the dense-mask fp32 specification on the host cores (S <= 8192)")
     p.add_argument("--model-patterns", action="store_true",
                    help="llm: also time block Scatter and window-with-sinks layers (g2s4 model setting)")
     p.add_argument("--backward", action="store_true", help="also time the backward pass (dq, dk, dv) of each pattern")
+    p.add_argument("--pattern", default="scatter",
+                   choices=["scatter", "gather1", "window", "image_scatter", "image_gather0"], help="phases: which kernel")
+    p.add_argument("--seqlen", type=int, default=32768, help="phases: LLM sequence length")
+    p.add_argument("--width", type=int, default=64, help="phases: image grid side")
+    p.add_argument("--softmax", default="auto", choices=["auto", "exact", "fast"], help="phases: softmax arithmetic")
     p.add_argument("--out", help="optional JSON output path")
     args = p.parse_args()
     args.seqlens = [int(x) for x in args.seqlens.split(",")]
     args.widths = [int(x) for x in args.widths.split(",")]
     args.groups = [int(x) for x in args.groups.split(",")]
     print(f"device: {torch.cuda.get_device_name()}  torch {torch.__version__}  peak {PEAK_BF16_TFLOPS} TFLOP/s")
-    rows = bench_llm(args) if args.mode == "llm" else bench_image(args)
+    rows = {"llm": bench_llm, "image": bench_image, "phases": bench_phases, "ceiling": bench_ceiling}[args.mode](args)
     if args.out:
         json.dump({"device": torch.cuda.get_device_name(), "torch": torch.__version__,
                    "args": {k: v for k, v in vars(args).items() if k != "out"}, "rows": rows},

@@ -1,0 +1,86 @@
+"""The benchmark driver (intra_amd/bench_kernel.py) against the reference's
+benchmarks/bench_kernel.py:52-111 and its published result files: same CLI, same JSON envelope,
+every row key of benchmarks/results/a100_llm.json / a100_image.json present with a positive
+latency, the reference's 32-layer arithmetic, and the added columns consistent with the latency
+and with the oracle's pair counts."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SCHEMA = json.load(open(os.path.join(ROOT, "tests", "golden", "reference_result_schema.json")))
+PEAK = 2516.6
+
+
+def run_cli(tmp_path, *argv, lib=None):
+    out = tmp_path / "rows.json"
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    if lib:
+        env["INTRA_HIP_LIB"] = lib
+    res = subprocess.run([sys.executable, "-m", "intra_amd.bench_kernel", *argv, "--out", str(out)], cwd=ROOT, env=env,
+                         capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0, res.stdout + res.stderr
+    doc = json.load(open(out))
+    for key in SCHEMA["envelope"] + ["torch"]:
+        assert key in doc, key
+    for key in SCHEMA["args"]:
+        assert key in doc["args"], key
+    return doc, res.stdout
+
+
+def test_llm_rows(tmp_path):
+    doc, _ = run_cli(tmp_path, "llm", "--seqlens", "1024,2048", "--iters", "3", "--warmup", "1", "--cpu")
+    assert doc["args"]["mode"] == "llm" and doc["args"]["seqlens"] == [1024, 2048] and doc["args"]["groups"] == [2, 8]
+    assert [r["seqlen"] for r in doc["rows"]] == [1024, 2048]
+    kinds = {"scatter_g2": ("llm/scatter", dict(group_num=2)), "scatter_g8": ("llm/scatter", dict(group_num=8)),
+             "gather1_g8": ("llm/gather1", dict(group_num=8)), "window576": ("llm/window", dict(window=576))}
+    for r in doc["rows"]:
+        for key in SCHEMA["llm_row"]:
+            assert key in r and r[key] > 0, key
+        S = r["seqlen"]
+        assert abs(r["g2s4_32layer"] - (4 * r["scatter_g2"] + 28 * r["window576"])) <= 2e-3
+        assert abs(r["dense_32layer"] - 32 * r["dense"]) <= 2e-3
+        assert r["g2s4_32layer_run"] > 0 and r["cpu_cores"] >= 1
+        for key, (kind, kw) in kinds.items():
+            flop = 4 * 128 * oracle.pairs_per_head(kind, S, **kw) * 32
+            tf = flop / (r[key] * 1e-3) / 1e12
+            assert abs(r[key + "_tflops"] - tf) <= 0.06 + 1e-3 * tf, key      # rounded to 0.1; ms rounded to 1e-4
+            assert abs(r[key + "_pct_peak"] - 100 * tf / PEAK) <= 0.06 + 1e-3 * tf
+            assert r[key + "_cpu_ms"] > r[key]      # the fp32 dense-mask specification on the host cores
+
+
+def test_image_rows(tmp_path):
+    doc, _ = run_cli(tmp_path, "image", "--widths", "64", "--iters", "3", "--warmup", "1", "--image-heads", "4", "--cpu")
+    (r,) = doc["rows"]
+    for key in SCHEMA["image_row"]:
+        assert key in r and r[key] > 0, key
+    assert r["width"] == 64 and r["seqlen"] == 4608
+    assert abs(r["interleaved_mean"] - (r["scatter"] + r["gather0"]) / 2) <= 1e-3
+    for key in ("scatter", "gather0"):
+        flop = 4 * 128 * oracle.pairs_per_head("image/" + key, 4608, width=64) * 4
+        tf = flop / (r[key] * 1e-3) / 1e12
+        assert abs(r[key + "_tflops"] - tf) <= 0.06 + 1e-3 * tf
+        assert r[key + "_cpu_ms"] > r[key]
+
+
+def test_ceiling_and_phases_modes(tmp_path):
+    doc, _ = run_cli(tmp_path, "ceiling")
+    const, rand = doc["rows"]
+    assert const["operands"].startswith("constant") and 0 < rand["tflops"] <= const["tflops"] * 1.02 <= PEAK * 1.05
+    assert 1000 < rand["shader_clock_mhz"] <= const["shader_clock_mhz"] * 1.02 < 2600
+    from intra_amd import _lib
+    doc, _ = run_cli(tmp_path, "phases", "--pattern", "scatter", "--seqlen", "8192", "--iters", "3", "--warmup", "1",
+                     lib=_lib.DIAG_LIB_PATH)
+    (r,) = doc["rows"]
+    assert r["workgroups"] == 256 and r["items_per_workgroup"] >= 1 and r["us_per_tile"] > 0
+    assert 0 < r["share_outside_tile_loop"] < 1 and all(v >= 0 for v in r["us_per_item"].values())
+    # the production library refuses the timer buffer instead of ignoring it
+    res = subprocess.run([sys.executable, "-m", "intra_amd.bench_kernel", "phases", "--seqlen", "1024"], cwd=ROOT,
+                         env=dict(os.environ, PYTHONPATH=ROOT), capture_output=True, text=True, timeout=300)
+    assert res.returncode != 0 and "INTRA_DIAG_TIMERS" in res.stdout + res.stderr
