@@ -150,6 +150,28 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
 int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int group_num,
                                 int window, int block, int offset, int n_sink);
 
+/* intra_llm_bwd for callers that cannot allocate device memory and have no workspace to hand
+ * over: code under HIP graph capture, tight serving or training loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference.  Same arguments and results as intra_llm_bwd
+ * without `workspace`: the kernels use an array of INTRA_NOALLOC_SCRATCH_FLOATS floats (16 MiB)
+ * that is part of the library's device image, one copy per GPU, held until the process ends.
+ * Calls whose intra_llm_bwd_workspace(...) exceeds that size return INTRA_ERR_UNSUPPORTED.  The
+ * entry point calls no hipMalloc / hipFree and no allocating library routine.  All calls on one
+ * GPU share that GPU's array: calls that overlap in time on one GPU (different streams or
+ * threads) race; calls on one stream, or otherwise ordered, are fine.  Nothing in the array has
+ * to survive between calls or start at zero: every value a launch reads was written by an earlier
+ * launch of the same call. */
+#define INTRA_NOALLOC_SCRATCH_FLOATS (4 * 1024 * 1024)
+int intra_llm_bwd_noalloc(const void* q, const void* k, const void* v, const void* o,
+                          const float* lse, const void* dout, void* dq, void* dk, void* dv, int B,
+                          int S, int H, int Hkv, const int64_t q_strides[3],
+                          const int64_t k_strides[3], const int64_t v_strides[3],
+                          const int64_t o_strides[3], const int64_t dout_strides[3],
+                          const int64_t dq_strides[3], const int64_t dk_strides[3],
+                          const int64_t dv_strides[3], const int64_t lse_strides[3], int pattern,
+                          int group_num, int window, int block, int offset, int n_sink,
+                          float softmax_scale, void* hip_stream);
+
 /* The same for intra_image_fwd: dq, dk, dv of image Scatter and Gather 0 (arguments as in
  * intra_llm_bwd; pattern, width, text_len as in intra_image_fwd).  dq in one launch; the grid keys'
  * dk / dv against the queries that see them (Scatter: their group's; Gather 0: the query patches

@@ -33,6 +33,8 @@ SYMBOLS = {
                                                ctypes.POINTER(ctypes.c_int64)]),
     "intra_llm_bwd": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 9 +
                       [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_void_p]),
+    "intra_llm_bwd_noalloc": (ctypes.c_int, [ctypes.c_void_p] * 9 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 9 +
+                              [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_void_p]),
     "intra_image_bwd": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 9 +
                         [ctypes.c_int] * 3 + [ctypes.c_float, ctypes.c_void_p]),
     "intra_image_bwd_workspace": (ctypes.c_int64, [ctypes.c_int] * 7),

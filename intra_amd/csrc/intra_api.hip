@@ -626,6 +626,31 @@ int run_bwd(int domain, const void* q, const void* k, const void* v, const void*
   }
 }
 
+// ------------------------------------------------------------------------------------ no-allocation backward
+// Workspace of intra_llm_bwd_noalloc: one array per GPU inside the library's own device image, so the
+// entry point never calls an allocator.  In host code the array's name only stands for the symbol; the
+// address the kernels get comes from hipGetSymbolAddress, asked once per device with that device current.
+static __device__ __align__(256) float scratch[INTRA_NOALLOC_SCRATCH_FLOATS];
+
+float* noalloc_scratch() {
+  static std::atomic<float*> ptrs[64];  // per device; nullptr = not asked yet
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
+    return nullptr;
+  }
+  float* ptr = ptrs[dev].load(std::memory_order_acquire);
+  if (ptr == nullptr) {
+    const hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      fail(INTRA_ERR_HIP, "hipGetSymbolAddress of the built-in workspace failed: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    ptrs[dev].store(ptr, std::memory_order_release);  // every thread gets the same answer for a device
+  }
+  return ptr;
+}
+
 // Host walk of the backward decomposition: count[q * S + k] += 1 for every (query, key) pair that
 // the dK / dV launches (key-row maps with their `store` rule, then the sink pass) multiply.
 template <class R>
@@ -740,6 +765,29 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
   return run_bwd(0, q, k, v, o, lse, dout, dq, dk, dv, workspace, B, S, H, Hkv, q_strides, k_strides, v_strides,
                  o_strides, dout_strides, dq_strides, dk_strides, dv_strides, lse_strides, pattern, group_num,
                  window, block, offset, n_sink, softmax_scale, hip_stream);
+}
+
+int intra_llm_bwd_noalloc(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
+                          void* dq, void* dk, void* dv, int B, int S, int H, int Hkv, const int64_t q_strides[3],
+                          const int64_t k_strides[3], const int64_t v_strides[3], const int64_t o_strides[3],
+                          const int64_t dout_strides[3], const int64_t dq_strides[3], const int64_t dk_strides[3],
+                          const int64_t dv_strides[3], const int64_t lse_strides[3], int pattern, int group_num,
+                          int window, int block, int offset, int n_sink, float softmax_scale, void* hip_stream) {
+  g_err[0] = 0;
+  Request r;
+  int rc = make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true);
+  if (rc) return rc;
+  if ((rc = bwd_supported(r))) return rc;
+  const int64_t need = bwd_workspace_floats(r);
+  if (need > (int64_t)INTRA_NOALLOC_SCRATCH_FLOATS)
+    return fail(INTRA_ERR_UNSUPPORTED,
+                "intra_llm_bwd_noalloc: this call needs %lld floats of workspace, the built-in one holds %lld; "
+                "use intra_llm_bwd with a workspace of the caller", (long long)need, (long long)INTRA_NOALLOC_SCRATCH_FLOATS);
+  float* work = noalloc_scratch();
+  if (work == nullptr) return INTRA_ERR_HIP;
+  return run_bwd(0, q, k, v, o, lse, dout, dq, dk, dv, work, B, S, H, Hkv, q_strides, k_strides, v_strides, o_strides,
+                 dout_strides, dq_strides, dk_strides, dv_strides, lse_strides, pattern, group_num, window, block, offset,
+                 n_sink, softmax_scale, hip_stream);
 }
 
 int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int group_num, int window, int block,
