@@ -375,8 +375,8 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
       return fail(INTRA_ERR_INVALID, "lse has a zero stride over a dimension larger than 1");
   }
 
-  if (ks[1] >= ((int64_t)1 << 31) || vs[1] >= ((int64_t)1 << 31))
-    return fail(INTRA_ERR_UNSUPPORTED, "k / v token stride must stay below 2^31 elements");
+  if (qs[1] >= ((int64_t)1 << 31) || ks[1] >= ((int64_t)1 << 31) || vs[1] >= ((int64_t)1 << 31))
+    return fail(INTRA_ERR_UNSUPPORTED, "q / k / v token stride must stay below 2^31 elements");
 
   intra::KParams p;
   p.q = static_cast<const uint16_t*>(q);
@@ -396,6 +396,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.q_fold = scale * 1.4426950408889634f;
   p.k_rs_bytes = (uint32_t)(ks[1] * 2);
   p.v_rs_bytes = (uint32_t)(vs[1] * 2);
+  p.q_rs_bytes = (uint32_t)(qs[1] * 2);
 
   Shape ph;
   if (!shape_for(r, default_hp(H / Hkv), &ph))

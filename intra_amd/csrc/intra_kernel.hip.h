@@ -21,7 +21,11 @@
 //    256-byte row, no register staging), three tiles ahead; one barrier per 64-key tile, which
 //    only waits for the requests of the previous iteration.  The tiles of all work items of a
 //    workgroup form one stream through the ring, so the first tiles of a work item arrive while
-//    the previous one still computes.  An LDS tile is 16 groups of 4 rows with an XOR chunk
+//    the previous one still computes.  The Q rows of a work item travel in the same stream, as
+//    two ring slots in front of its key tiles: they are requested three slots ahead like any
+//    tile, arrive as whole 256-byte rows, and each wavefront picks its 32 rows out of LDS with
+//    the K operand's read pattern.  The output rows of a finished item stay in registers until
+//    the next item's first requests are out and are stored behind them.  An LDS tile is 16 groups of 4 rows with an XOR chunk
 //    swizzle inside the group and 16 bytes of padding between groups, so the row-per-lane K reads
 //    and the 4-row transposing V reads are both free of bank conflicts.
 //  * The softmax reference stays 0 (weights exp2(score*c), exact after normalisation because
@@ -73,7 +77,7 @@ struct KParams {
   float scale_log2;    // |softmax_scale| * log2(e)
   int negate_q;        // softmax_scale < 0: flip the sign of Q instead
   float q_fold;        // FAST mode: softmax_scale * log2(e), signed, multiplied into Q
-  uint32_t k_rs_bytes, v_rs_bytes;  // token strides of k and v in bytes (< 4 GiB, checked on the host)
+  uint32_t k_rs_bytes, v_rs_bytes, q_rs_bytes;  // token strides of k, v, q in bytes (< 4 GiB, checked on the host)
   int n_sets;          // sets per (batch, kv head)
   int n_mblocks;       // row blocks of the largest set
   int hgroups;         // ratio / HP
@@ -220,35 +224,58 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   static_assert((BN / 4) % NW == 0, "tile groups must split evenly over the wavefronts");
   const int ld_row = lane >> 4;                                  // row of the group this lane fetches
   const uint32_t ld_col = (((lane & 15) ^ (4 * ld_row)) << 4);   // byte column it fetches
-  const uint32_t k_rs_b = p.k_rs_bytes, v_rs_b = p.v_rs_bytes;
+  const uint32_t k_rs_b = p.k_rs_bytes, v_rs_b = p.v_rs_bytes, q_rs_b = p.q_rs_bytes;
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+  // The stream of a work item: slots -2 and -1 carry its 256 Q rows (wavefront w reads rows
+  // 32 * (w % 2) .. of the K part (w / 2 even) or V part (w / 2 odd) of slot w / 4), slots 0 .. ntiles-1
+  // its key tiles.
+  static_assert(NW == 8, "the Q slots are laid out for 8 wavefronts");
   struct Feed {
     MAP map;
     Range rg;
-    int nk, tile;
+    int nk, tile;      // tile: -2, -1 (Q slots), then the key tile being requested next
     bool more;         // false once the last work item has been requested completely
-    const char *kbase, *vbase;
-    Where w;           // the work item whose tiles are being requested
+    const char *kbase, *vbase, *qbase;
+    int t0, t1;        // first and last in-set query of the row block
+    Where w;           // the work item whose slots are being requested
     int prev_round;    // round of the work item before it
   };
   auto feed_for = [&](const Where& w, int prev_round) {
     const MAP map(p.geom, w.set, w.mblk * POS);
-    return Feed{map, range_of(map, w.mblk), map.nk(), 0, true,
+    return Feed{map, range_of(map, w.mblk), map.nk(), -2, true,
                 reinterpret_cast<const char*>(p.k + w.batch * p.k_bs + w.kvh * p.k_hs),
-                reinterpret_cast<const char*>(p.v + w.batch * p.v_bs + w.kvh * p.v_hs), w, prev_round};
+                reinterpret_cast<const char*>(p.v + w.batch * p.v_bs + w.kvh * p.v_hs),
+                reinterpret_cast<const char*>(p.q + w.batch * p.q_bs + (int64_t)(w.kvh * p.ratio + w.hg * HP) * p.q_hs),
+                w.mblk * POS, im_min(w.mblk * POS + POS, map.nq()) - 1, w, prev_round};
   };
   Where cw;
   if (!locate(0, cw)) return;
   INTRA_DIAG(long long dg[DIAG_SLOTS] = {0, 0, 0, 0, 0, 0, 0, 0};)
   Feed fd = feed_for(cw, -1);
-  auto feed_tile = [&](int slot_off) {  // request the next K and V tile of the stream into a ring slot
+  auto feed_tile = [&](int slot_off) {  // request the next slot of the stream into a ring slot
+    if (fd.tile < 0) {  // 128 Q rows: rows of four wavefronts, two per part
 #pragma unroll
-    for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
-      const int grp = wave * GROUPS_PER_WAVE + gi;
-      const int tk = im_min(fd.rg.kt_lo + fd.tile * BN + 4 * grp + ld_row, fd.nk - 1);
-      const uint32_t pos = fd.map.kpos(tk);
-      dma_group(fd.kbase + ((uint64_t)pos * k_rs_b + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
-      dma_group(fd.vbase + ((uint64_t)pos * v_rs_b + ld_col), lds_base + VBASE + slot_off + grp * GROUP_STRIDE);
+      for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
+        const int grp = wave * GROUPS_PER_WAVE + gi;
+        const int rho = 4 * grp + ld_row;  // row of the part
+#pragma unroll
+        for (int part = 0; part < 2; ++part) {
+          const int wq = (fd.tile + 2) * 4 + part * 2 + (rho >> 5);  // the wavefront that will read this row
+          const int t = im_min(fd.t0 + (wq / HP) * 32 + (rho & 31), fd.t1);
+          const uint32_t pos = fd.map.qpos(t);
+          dma_group(fd.qbase + ((int64_t)(wq % HP) * p.q_hs * 2 + (uint64_t)pos * q_rs_b + ld_col),
+                    lds_base + part * VBASE + slot_off + grp * GROUP_STRIDE);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
+        const int grp = wave * GROUPS_PER_WAVE + gi;
+        const int tk = im_min(fd.rg.kt_lo + fd.tile * BN + 4 * grp + ld_row, fd.nk - 1);
+        const uint32_t pos = fd.map.kpos(tk);
+        dma_group(fd.kbase + ((uint64_t)pos * k_rs_b + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
+        dma_group(fd.vbase + ((uint64_t)pos * v_rs_b + ld_col), lds_base + VBASE + slot_off + grp * GROUP_STRIDE);
+      }
     }
     ++fd.tile;
     if (fd.tile == fd.rg.ntiles && fd.more) {
@@ -257,7 +284,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
       else fd.more = false;  // nothing left: keep requesting the (clamped) last row, nobody reads it
     }
   };
-  constexpr int PER_TILE = 2 * GROUPS_PER_WAVE;  // requests per wavefront per tile (K + V)
+  constexpr int PER_TILE = 2 * GROUPS_PER_WAVE;  // requests per wavefront per slot (K + V parts)
 
   // LDS operand addresses.  With the chunk swizzle c ^ 4i of a group, the 16-byte chunk 2*ks + h32
   // of key row l32 (the K operand of k-step ks = 2a + b) sits at byte 64 * (a ^ r) + 32 * b +
@@ -281,13 +308,12 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   }
   // Q^T fragments: lane holds query l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
   bf16x8 qf[8];
-  // Q is fetched, and O stored, 64 contiguous bytes per row and instruction instead of 32: the two
-  // lanes of neighbouring queries 2a, 2a+1 (and their upper-half twins) together cover chunks
-  // 4m..4m+3 of row 2a in access 2m and of row 2a+1 in access 2m+1, lane (e = query parity, h)
-  // taking chunk 4m + 2e + h.  A lane then holds its own chunks 2ks + h only for ks = e (mod 2);
-  // the others sit in its neighbour and are swapped in with one quad permute per dword
-  // (pair_exchange, its own inverse).  Rows past the end of the row block are clamped to its
-  // last row.
+  auto kread_q = [&](int base, int off) { return *reinterpret_cast<const bf16x8*>(smem + (base + off)); };
+  // O is stored 64 contiguous bytes per row and instruction instead of 32: the two lanes of
+  // neighbouring queries 2a, 2a+1 (and their upper-half twins) together cover chunks 4m..4m+3 of
+  // row 2a in access 2m and of row 2a+1 in access 2m+1, lane (e = query parity, h) taking chunk
+  // 4m + 2e + h.  A lane holds its own chunks 2ks + h for every ks; those with ks != e (mod 2) are
+  // swapped with its neighbour's, one quad permute per dword (pair_exchange).
   const int qpar = l32 & 1;
   auto pair_exchange = [&](u32x4 (&r)[8]) {
 #pragma unroll
@@ -300,27 +326,45 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
         r[2 * m + 1][d] = qpar ? x1 : got;
       }
   };
-  auto load_q = [&](const Where& w) {
-    const MAP map(p.geom, w.set, w.mblk * POS);
-    const int t1 = im_min(w.mblk * POS + POS, map.nq()) - 1;
-    const int r0 = w.mblk * POS + (wave / HP) * 32 + (l32 & ~1);
-    const int hq = w.kvh * p.ratio + w.hg * HP + wave % HP;
-    const int64_t head = w.batch * p.q_bs + hq * p.q_hs + (2 * qpar + h32) * 8;
-    const uint16_t* row_a = p.q + (head + (int64_t)map.qpos(im_min(r0, t1)) * p.q_rs);
-    const uint16_t* row_b = p.q + (head + (int64_t)map.qpos(im_min(r0 + 1, t1)) * p.q_rs);
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-      qf[i] = *reinterpret_cast<const bf16x8*>(((i & 1) ? row_b : row_a) + 32 * (i >> 1));
-  };
 
   // Ring slots (byte offsets into the K ring; the V ring uses the same offsets behind VBASE) of
   // the stream tiles i, i+1, i+2, i+3 seen from the computation; they rotate once per tile and
   // carry on from one work item to the next.
   int k0 = 0, k1 = KTILE, k2 = 2 * KTILE, k3 = 3 * KTILE;
-  feed_tile(k0);
+  feed_tile(k0);  // the two Q slots of the first work item and its first key tile
   feed_tile(k1);
   feed_tile(k2);
-  load_q(cw);  // after the tile requests: the load counter is in order, so Q arrives last
+  auto rotate = [&] {  // one slot further in the stream
+    const int dk = k2 - k1, dv = k1 - k0;  // +KTILE, or -3 * KTILE where the ring wraps
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      kb[a] += dk;
+      vb[a] += dv;
+    }
+    const int tk = k0;
+    k0 = k1; k1 = k2; k2 = k3; k3 = tk;
+  };
+  // Barrier in front of a slot, leaving this wavefront's requests for the slot after the next in
+  // flight (the PER_TILE most recent operations) and, where they were issued in between, the
+  // `extra` stores of the previous work item's output (0, 8 or 9; wave-uniform).  The operation
+  // counter retires in issue order, so everything older than what is left pending has landed.
+  auto slot_barrier = [&](int extra) {
+    if (extra == 0) tile_barrier<PER_TILE>();
+    else if (extra == 8) tile_barrier<PER_TILE + 8>();
+    else tile_barrier<PER_TILE + 9>();
+  };
+  // Output of the finished work item, kept in registers until the next item's first requests are out
+  u32x4 pk[8];
+  uint16_t *orow_a = nullptr, *orow_b = nullptr;
+  float* lse_dst = nullptr;
+  float lse_val = 0.f;
+  int held = 0;  // vector-memory operations the held output will take: 0 (nothing held), 8, or 9 with a log-sum-exp
+  auto store_held = [&] {
+    if (held == 0) return;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(((i & 1) ? orow_b : orow_a) + 32 * (i >> 1)) = pk[i];
+    if (held == 9) *lse_dst = lse_val;
+  };
 
   for (;;) {
   INTRA_DIAG(const long long t_a = wall_clock64();)
@@ -362,21 +406,26 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
 
   const int hq = kvh * p.ratio + hg * HP + hw;
   const int64_t qpos = map.qpos(tq);
-  // the two rows this lane stores parts of (see load_q), and whether they exist
+  // The two rows this lane stores parts of.  Rows past the end of the row block are clamped to its
+  // last row, for Q and for O alike: such lanes compute that row once more and store the same
+  // bytes to the same place, so every active wavefront issues all of its stores.
   const int ra = wq0 + (l32 & ~1);
   const int64_t opos_a = map.qpos(im_min(ra, t1)), opos_b = map.qpos(im_min(ra + 1, t1));
-  const bool valid_a = ra <= t1, valid_b = ra + 1 <= t1;
-  // Pin the arrival of Q here: the empty asm uses and redefines the fragments, so the compiler waits
-  // for their loads at this point (where the wait is needed anyway) and not, with a counter value
-  // that also covers the tile requests in flight, in front of every MFMA that reads them.
+
+  // ---------------------------------------------------------------- slot -2: the Q rows arrive
+  INTRA_DIAG(const long long t_b = wall_clock64();)
+  tile_barrier<PER_TILE>();  // both Q slots have landed; the held stores are not out yet
+  INTRA_DIAG(const long long t_c = wall_clock64();)
+  feed_tile(k3);
+  store_held();              // behind the request, so that two more barriers can leave them in flight
+  const int in_flight = held;
+  held = 0;
   {
+    // this wavefront's 32 rows: slot wave / 4 (k0 or k1), part (wave / 2) % 2, rows 32 * (wave % 2) ..
+    const int qoff = ((wave >> 2) ? 0 : k0 - k1) + ((wave >> 1) & 1) * VBASE + (wave & 1) * BLOCK32;
     u32x4 raw[8];
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      raw[ks] = __builtin_bit_cast(u32x4, qf[ks]);
-      asm volatile("" : "+v"(raw[ks]));
-    }
-    pair_exchange(raw);
+    for (int g = 0; g < 8; ++g) raw[g] = __builtin_bit_cast(u32x4, kread_q(kb[g >> 1] + qoff, 32 * (g & 1)));
     if (FAST) {  // Q <- bf16(Q * softmax_scale * log2 e): the MFMA then yields exponents directly
       const float cq = p.q_fold;
 #pragma unroll
@@ -391,6 +440,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = __builtin_bit_cast(bf16x8, raw[ks]);
   }
+  rotate();
   if (!FAST && p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks)
@@ -597,66 +647,61 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   // may still be in flight.  Iteration i requests tile i+3 into the slot of tile i-1, which no
   // wavefront reads after the barrier that opened iteration i.  The barrier that opens iteration
   // i+1 only waits for the older requests, so every row has a whole iteration to arrive.
-  // At the start of a work item a wavefront has issued, after the requests for tiles 0 and 1:
-  // those for tile 2, its own Q (8 loads) and, unless it was idle, the output rows of the
-  // previous item (8 stores).  Letting PER_TILE + 8 operations pending is safe in both cases.
-  INTRA_DIAG(const long long t_b = wall_clock64();)
-  tile_barrier<PER_TILE + 8>();
-  INTRA_DIAG(const long long t_c = wall_clock64();)
-  if (jq1 < 0 && jp1 >= 0) {
-    load_ka(ka, k0 - k1, 0);
+  // The two Q slots in front of a work item's tiles are iterations of the same kind without
+  // tile work: the first reads Q out of LDS, the second computes the scores of key block 0.
+  // ---------------------------------------------------------------- slot -1: the first key tile has landed
+  slot_barrier(in_flight);
+  feed_tile(k3);
+  if (jq1 < 0 && jp1 >= 0) {  // scores of key block 0, ahead of the pipeline (the tile sits in slot k1)
+    load_ka(ka, 0, 0);
     s0 = zero16();
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qf[ks], s0, 0, 0, 0);
     finish_scores(s0, FAST ? 0.f : block_max(s0), needs_mask(0), kt_lo);
-    load_ka(ka, k0 - k1, BLOCK32);
+    load_ka(ka, 0, BLOCK32);
   }
+  rotate();
   INTRA_DIAG(const long long t_d = wall_clock64(); const long long c_d = __builtin_readcyclecounter();)
-  for (int i = 0; i < ntiles; ++i) {
-    if (i > 0) tile_barrier<PER_TILE>();
+  slot_barrier(in_flight);  // opens tile 0; the held stores went out after the request for tile 1
+  for (int i = 0;;) {
     step(2 * i, s0, s1, ic<0>{}, ic<1>{}, k3);
     step(2 * i + 1, s1, s0, ic<BLOCK32>{}, ic<0>{}, 0);
-    const int dk = k2 - k1, dv = k1 - k0;  // +KTILE, or -3 * KTILE where the ring wraps
-#pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      kb[a] += dk;
-      vb[a] += dv;
-    }
-    const int tk = k0;
-    k0 = k1; k1 = k2; k2 = k3; k3 = tk;
+    rotate();
+    if (++i == ntiles) break;
+    tile_barrier<PER_TILE>();
   }
 
   INTRA_DIAG(const long long t_e = wall_clock64(); dg[7] += __builtin_readcyclecounter() - c_d;)
-  // Q of the next work item is requested before the output rows of this one are stored, so that
-  // it travels while the epilogue runs (qf is dead here).
-  // The loader is ahead by three tiles, so it usually knows the next work item already.
+  // The loader is ahead by three slots, so it usually knows the next work item already.
   Where nw = fd.w;
   bool more = true;
   if (fd.w.round == cw.round) more = false;  // (the loader only stays on an item when it is the last)
   else if (fd.prev_round != cw.round) more = locate(cw.round + 1, nw);
-  if (more) load_q(nw);
 
-  // ---------------------------------------------------------------- normalise and scatter-store
-  if (wave_active) {
+  // ---------------------------------------------------------------- normalise; the rows are stored later
+  // (idle wavefronts run through it as well and hold nothing: the registers of the held output
+  // are then rewritten in every work item and free during the tile loop)
+  {
   const float l_tot = lane_xor32_sum(l_acc[0] + l_acc[1]);
   if (FAST) {
     // Weights were formed without a reference: the result is good iff the weight sum stayed inside
     // 2^-100 .. 2^60 (no weight overflowed, and the largest ones are far from underflow).  The
     // integer comparison of the bit patterns also catches a negative or NaN sum.
     const uint32_t lb = __float_as_uint(l_tot);
-    const bool bad = row_valid && !(lb >= 0x0d800000u && lb <= 0x5d800000u);
+    const bool bad = wave_active && row_valid && !(lb >= 0x0d800000u && lb <= 0x5d800000u);
     if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0)
       __hip_atomic_fetch_or(&redo[(cw.round >> 5) & (REDO_WORDS - 1)], 1u << (cw.round & 31), __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_WORKGROUP);
   }
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (p.lse != nullptr && row_valid && h32 == 0)  // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2
-    p.lse[batch * p.lse_bs + hq * p.lse_hs + qpos * p.lse_ts] = (mref + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+  // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2; lanes of clamped rows repeat their row's value
+  held = wave_active ? (p.lse != nullptr ? 9 : 8) : 0;
+  lse_dst = p.lse + (batch * p.lse_bs + hq * p.lse_hs + qpos * p.lse_ts);
+  lse_val = (mref + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   // Lane l and lane l+32 hold the same query: per 16 head dims the lower lane has dims 0-3 and
   // 8-11, the upper one 4-7 and 12-15.  One permlane32 swap per register pair turns that into
   // dims 0-7 / 8-15, i.e. 16-byte chunk 2*ks + h of the row for ks = 2*db + g2; pair_exchange
   // then regroups the chunks so that four lanes store 64 contiguous bytes of one row.
-  u32x4 pk[8];
 #pragma unroll
   for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -676,19 +721,15 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     }
   pair_exchange(pk);
   const int64_t ohead = batch * p.o_bs + hq * p.o_hs + (2 * qpar + h32) * 8;
-  uint16_t* orow_a = p.o + (ohead + opos_a * p.o_rs);
-  uint16_t* orow_b = p.o + (ohead + opos_b * p.o_rs);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    if ((i & 1) ? valid_b : valid_a)
-      *reinterpret_cast<u32x4*>(((i & 1) ? orow_b : orow_a) + 32 * (i >> 1)) = pk[i];
-  }
+  orow_a = p.o + (ohead + opos_a * p.o_rs);
+  orow_b = p.o + (ohead + opos_b * p.o_rs);
   }
   INTRA_DIAG(dg[0] += t_b - t_a; dg[1] += t_c - t_b; dg[2] += t_d - t_c; dg[3] += t_e - t_d;
              dg[4] += wall_clock64() - t_e; dg[5] += 1; dg[6] += ntiles;)
   if (!more) break;
   cw = nw;
   }  // work items
+  store_held();
   INTRA_DIAG(if (p.diag != nullptr && tid == 0) for (int i = 0; i < DIAG_SLOTS; ++i)
                p.diag[(size_t)blockIdx.x * DIAG_SLOTS + i] += dg[i];)
 }
