@@ -88,4 +88,5 @@ def _strides_array(s0, s1, s2):
 def strides3(x):
     """The first three element strides of a tensor ((batch, token, head) of a (B, S, H, D) tensor)
     as a C array; the arrays are read-only for the library and cached."""
-    return _strides_array(x.stride(0), x.stride(1), x.stride(2))
+    st = x.stride()
+    return _strides_array(st[0], st[1], st[2])

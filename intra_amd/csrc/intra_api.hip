@@ -330,6 +330,44 @@ bool use_fast_softmax(float scale) {
   return fabsf(scale) <= INTRA_FAST_SOFTMAX_MAX_SCALE;
 }
 
+// Order of an XCD's work items (see KParams::Section).  One section - every pair, all row blocks - except
+// where a launch mixes full-size items with items that keep only a quarter of the workgroup busy:
+//  * image scatter: a set has text_len / 8 + width^2 / 8 queries, so its last row block is partial
+//    (64 of 256 rows at 24 heads); those row blocks of all pairs form a second section;
+//  * image gather0: the text-only sets (64 queries each, against text + one group's grid keys) and
+//    the patch runs (256 queries against text + window keys); whichever kind takes longer goes first.
+void set_sections(intra::KParams& p, const Request& r, const Shape& ph, const LaunchDims& d) {
+  const int pslots = (d.n_pairs + 7) / 8;
+  auto section = [&](int p_lo, int p_n, int mb_lo, int mb_hi) {
+    intra::KParams::Section s;
+    s.p_lo = p_lo;
+    s.mb_hi = mb_hi;
+    s.slots = p_n * (mb_hi - mb_lo) * d.hgroups;
+    s.d_ipp = make_fastdiv(std::max(1, (mb_hi - mb_lo) * d.hgroups));
+    return s;
+  };
+  p.sec[0] = section(0, pslots, 0, d.n_mblocks);
+  p.sec[1] = section(0, 0, 0, 1);
+  if (ph.map == MAP_IMG_SCATTER) {
+    const int nq = r.geom.text_len / 8 + r.geom.width * r.geom.width / 8;
+    if (d.n_mblocks >= 2 && nq % d.pos != 0 && 2 * (nq % d.pos) <= d.pos) {
+      p.sec[0] = section(0, pslots, 0, d.n_mblocks - 1);
+      p.sec[1] = section(0, pslots, d.n_mblocks - 1, d.n_mblocks);
+    }
+  } else if (ph.map == MAP_IMG_GATHER0) {
+    // pairs are numbered set-major, so the 8 text sets are the pair slots below B * Hkv
+    const int text_slots = r.B * r.Hkv;
+    const int64_t text_keys = r.geom.text_len + (int64_t)r.geom.width * r.geom.width / 8;
+    const int64_t patch_keys = r.geom.text_len + 16 * (16 + 8 * (ph.geom.pg - 1));
+    // a text item keeps 2 of 8 wavefronts busy and runs a key tile in about 2/3 of the time
+    if (3 * patch_keys > 2 * text_keys && pslots > text_slots) {
+      p.sec[0] = section(text_slots, pslots - text_slots, 0, d.n_mblocks);
+      p.sec[1] = section(0, text_slots, 0, d.n_mblocks);
+    }
+  }
+  p.n_slots = p.sec[0].slots + p.sec[1].slots;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // `written`: the tensor is an output, so its elements may not alias (a zero stride over a dimension
@@ -412,9 +450,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.n_mblocks = dims.n_mblocks;
   p.hgroups = dims.hgroups;
   p.n_pairs = dims.n_pairs;
-  p.items_per_pair = dims.hgroups * dims.n_mblocks;
-  p.n_slots = dims.work_items / 8;
-  p.d_items_per_pair = make_fastdiv(p.items_per_pair);
+  set_sections(p, r, ph, dims);
   p.d_nbh = make_fastdiv(B * Hkv);
   p.d_hkv = make_fastdiv(Hkv);
   p.d_hgroups = make_fastdiv(p.hgroups);

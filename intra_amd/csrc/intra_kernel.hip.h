@@ -82,9 +82,17 @@ struct KParams {
   int n_mblocks;       // row blocks of the largest set
   int hgroups;         // ratio / HP
   int n_pairs;         // B * Hkv * n_sets
-  int items_per_pair;  // hgroups * n_mblocks
-  int n_slots;         // work items per XCD: ceil(n_pairs / 8) * items_per_pair
-  FastDiv d_items_per_pair, d_nbh, d_hkv, d_hgroups;  // divisions by items_per_pair, B * Hkv, Hkv, hgroups
+  int n_slots;         // work items per XCD: sum of the sections' slots
+  // The work items of an XCD are numbered section by section (costly kinds of items first, so
+  // that the cheap ones fill the last, partial round of the workgroups): a section is a range of
+  // the XCD's pairs times a range of row blocks, taken pair by pair, last row block first.
+  struct Section {
+    int p_lo;          // first pair slot (pair = 8 * pair slot + XCD)
+    int mb_hi;         // one past its last row block
+    int slots;         // pair slots * row blocks * hgroups
+    FastDiv d_ipp;     // division by its items per pair: row blocks * hgroups
+  } sec[2];
+  FastDiv d_nbh, d_hkv, d_hgroups;  // divisions by B * Hkv, Hkv, hgroups
   long long* diag;     // INTRA_DIAG_TIMERS builds: DIAG_SLOTS counters per workgroup, or null
 };
 
@@ -182,17 +190,20 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
       const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
       if (slot >= p.n_slots) return false;
       if (REDO && !((redo[(round >> 5) & (REDO_WORDS - 1)] >> (round & 31)) & 1u)) continue;
-      const int pslot = (int)fd_div(slot, p.d_items_per_pair);
-      const int pair = pslot * 8 + xcd;
+      const bool second = slot >= p.sec[0].slots;
+      const KParams::Section& sc = p.sec[second ? 1 : 0];
+      const int sslot = second ? slot - p.sec[0].slots : slot;
+      const int pq = (int)fd_div(sslot, sc.d_ipp);
+      const int pair = (sc.p_lo + pq) * 8 + xcd;
       if (pair >= p.n_pairs) continue;
-      const int rem = slot - pslot * p.items_per_pair;
+      const int rem = sslot - pq * (int)sc.d_ipp.d;
       const int rblk = (int)fd_div(rem, p.d_hgroups);
       w.round = round;
       w.set = (int)fd_div(pair, p.d_nbh);
       const int bh = pair - w.set * (int)p.d_nbh.d;
       w.batch = (int)fd_div(bh, p.d_hkv);
       w.kvh = bh - w.batch * p.Hkv;
-      w.mblk = p.n_mblocks - 1 - rblk;
+      w.mblk = sc.mb_hi - 1 - rblk;
       w.hg = rem - rblk * p.hgroups;
       if (w.mblk * POS >= MAP(p.geom, w.set, w.mblk * POS).nq()) continue;
       return true;

@@ -25,7 +25,12 @@ TEXT_LEN = 512
 
 
 def _aligned(x):
-    return x.stride(-1) == 1 and x.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in x.stride()[:-1])
+    if x.data_ptr() % 16:
+        return False
+    if x.is_contiguous():  # the usual case, and the cheap test: rows of 128 bf16 are 256 bytes
+        return True
+    st = x.stride()
+    return st[-1] == 1 and st[0] % 8 == 0 and st[1] % 8 == 0 and st[2] % 8 == 0
 
 
 SOFTMAX_MODES = {"auto": 0, "exact": 1, "fast": 2}
@@ -69,9 +74,15 @@ def _scale(q, softmax_scale):
 def _stream_on(device):
     """(context that makes `device` current, handle of its current stream).  Switching devices is
     only paid for when the tensors live on another GPU than the current one."""
-    if device.index == torch.cuda.current_device():
-        return contextlib.nullcontext(), torch.cuda.current_stream().cuda_stream
-    return torch.cuda.device(device), torch.cuda.current_stream(device).cuda_stream
+    index = device.index
+    if index == torch.cuda.current_device():
+        return _NO_GUARD, _raw_stream(index)
+    return torch.cuda.device(device), _raw_stream(index)
+
+
+_NO_GUARD = contextlib.nullcontext()
+# handle of the current stream of a device without building a torch.cuda.Stream object per call
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (lambda i: torch.cuda.current_stream(i).cuda_stream)
 
 
 def _launch(fn, fn_lse, q, k, v, pattern_id, arg0, arg1, scale, return_lse=False):
@@ -79,16 +90,17 @@ def _launch(fn, fn_lse, q, k, v, pattern_id, arg0, arg1, scale, return_lse=False
     if not _aligned(out):
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     B, S, H, _ = q.shape
-    args = [q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
-            _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
-            pattern_id, arg0, arg1, float(scale)]
-    lse = torch.empty(B, H, S, dtype=torch.float32, device=q.device) if return_lse else None
     guard, stream = _stream_on(q.device)
     with guard:
         if return_lse:
-            rc = fn_lse(*args, stream, lse.data_ptr(), _lib.strides3(lse))
+            lse = torch.empty(B, H, S, dtype=torch.float32, device=q.device)
+            rc = fn_lse(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
+                        _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                        pattern_id, arg0, arg1, float(scale), stream, lse.data_ptr(), _lib.strides3(lse))
         else:
-            rc = fn(*args, stream)
+            rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
+                    _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                    pattern_id, arg0, arg1, float(scale), stream)
     if rc != _lib.INTRA_OK:
         raise RuntimeError(f"intra_hip: {_lib.last_error()}")
     return (out, lse) if return_lse else out
