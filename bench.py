@@ -20,9 +20,21 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/clk/CU; AMD publishes it as 2.5 PFLOP/s dense
-# HBM bytes per launch at S=32768 measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/); None until measured for the current kernel.
-MEASURED_TRAFFIC_BYTES = {32768: 793e6}
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, written by
+# `python -m intra_amd.rocprof_summary traffic` together with a hash of the kernel sources
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(seqlen):
+    """Bytes per launch if they were measured for exactly this kernel source and workload, else None."""
+    try:
+        from intra_amd.rocprof_summary import source_hash
+        rec = json.load(open(TRAFFIC_FILE))
+        if rec.get("source_sha256_16") == source_hash() and rec.get("seqlen") == seqlen:
+            return rec["hbm_bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        pass
+    return None
 
 
 def main():
@@ -70,6 +82,14 @@ def main():
 
     step = lambda: intra_llm_attn(q, k, v, "scatter", group_num=G)
     with torch.no_grad():
+        # parity spot check on a row subset first, so that a wrong kernel cannot post a number (it also
+        # brings the clocks up before the warm-up steps)
+        out = step()
+        rows = torch.unique(torch.cat([torch.randperm(S, generator=g)[:256], torch.tensor([0, S - 1])])).to(dev)
+        ref = oracle.masked_attention_rows(q, k, v, oracle.llm_scatter_mask(S, G, dev, rows), rows)
+        err = (out[:, rows].float() - ref.float()).abs().max().item()
+        assert err <= 1.6e-2, f"parity failed in bench: {err}"
+        del ref
         for _ in range(args.warmup):
             out = step()
         torch.cuda.synchronize()
@@ -90,11 +110,8 @@ def main():
         kern_ms = sorted(a.elapsed_time(b) for a, b in evs)
     kern_avg = sum(kern_ms) / len(kern_ms)
 
-    # parity spot check on a row subset so that a wrong kernel cannot post a number
-    rows = torch.unique(torch.cat([torch.randperm(S, generator=g)[:256], torch.tensor([0, S - 1])])).to(dev)
-    ref = oracle.masked_attention_rows(q, k, v, oracle.llm_scatter_mask(S, G, dev, rows), rows)
-    err = (out[:, rows].float() - ref.float()).abs().max().item()
-    assert err <= 1.6e-2, f"parity failed in bench: {err}"
+    # the timed launches must have produced the same output as the checked one
+    assert torch.equal(out, step()), "output changed between launches"
 
     tflops = flop / (wall_ms * 1e-3) / 1e12
     achieved = flop / (kern_avg * 1e-3) / 1e12
@@ -112,7 +129,7 @@ def main():
         "parity_max_abs_err": err, "softmax": args.softmax,
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(S)},
+                     "traffic": measured_traffic(S)},
         "device": torch.cuda.get_device_name(0),
         "cu_count": torch.cuda.get_device_properties(0).multi_processor_count,
     }
@@ -154,6 +171,29 @@ def main():
                 b.record()
                 torch.cuda.synchronize()
                 gpu_ms.append(a.elapsed_time(b))
+        # like for like: the whole problem at the headline's head layout (32 query / 8 kv heads) at the
+        # largest length the dense-mask path handles in seconds, CPU and GPU on the same inputs
+        Sw = min(S, 8192)
+        qw, kw_, vw = (t[:, :Sw].contiguous() for t in (q_cpu, k_cpu, v_cpu))
+        mask_w = oracle.llm_scatter_mask(Sw, G)
+        t0 = time.perf_counter()
+        oracle.masked_attention(qw, kw_, vw, mask_w, chunk=512)
+        cpu_s = time.perf_counter() - t0
+        qg, kg, vg = qw.to(dev), kw_.to(dev), vw.to(dev)
+        gpu_ms = []
+        with torch.no_grad():
+            for i in range(13):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                intra_llm_attn(qg, kg, vg, "scatter", group_num=G)
+                b.record()
+                torch.cuda.synchronize()
+                gpu_ms.append(a.elapsed_time(b))
+        eff_w = 4.0 * 128 * oracle.pairs_per_head("llm/scatter", Sw, group_num=G) * H * B
+        res["cpu_baseline"]["whole_problem"] = {
+            "workload": f"LLM causal Scatter G={G}, B=1, S={Sw}, {H} query / {Hkv} kv heads",
+            "cpu_ms": round(cpu_s * 1e3, 1), "cpu_tflops_effective": round(eff_w / cpu_s / 1e12, 6),
+            "gpu_ms": round(sorted(gpu_ms[3:])[5], 4)}
         res["cpu_baseline"]["small_case"] = {
             "workload": f"LLM causal Scatter G={G}, B=1, S=1024, 4 query / 1 kv heads",
             "cpu_ms": round(sorted(cpu_ms[1:])[2], 3), "gpu_ms": round(sorted(gpu_ms[3:])[2], 4)}

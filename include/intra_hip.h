@@ -145,7 +145,8 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
                   int offset, int n_sink, float softmax_scale, void* hip_stream);
 /* Floats of workspace that intra_llm_bwd needs for such a call (B*H*S rounded up to 4, plus with
  * sinks chunks * B * Hkv * min(n_sink, S) * 128, the queries being cut into chunks so that the
- * sink pass has about one workgroup per CU); -1 if the request is invalid or unsupported
+ * sink pass has about one workgroup per CU; the size is the same on every device - it allows for
+ * 320 CUs, and a launch never splits finer than that); -1 if the request is invalid or unsupported
  * (intra_last_error() says why).  No counterpart in the reference. */
 int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int group_num,
                                 int window, int block, int offset, int n_sink);
@@ -204,7 +205,7 @@ typedef struct IntraPlan {
   int work_items;      /* row blocks to process, all launches (a multiple of 8: padded per XCD) */
   int grid;            /* upper bound of workgroups launched: min(work_items, CUs of the device) */
   int lds_bytes;       /* LDS per workgroup */
-  int launches;        /* kernel launches per call (1 for every pattern of this build) */
+  int launches;        /* kernel launches per forward call: 1 for every pattern */
   int64_t pairs_per_head; /* unmasked (query, key) pairs per query head and batch */
 } IntraPlan;
 

@@ -266,9 +266,9 @@ template <class MAP> struct ModelWalk {
   static int go(const IntraGeom& ge, int hp, int nw, uint8_t* count) { model_walk<MAP>(ge, hp, nw, count); return 0; }
 };
 
-// One persistent workgroup per CU (LDS allows no more), in multiples of the 8 XCDs.
-int launch_grid(int work_items) {
-  static std::atomic<int> cus[64];  // CU count per device, 0 = not asked yet (same answer from every thread)
+// CUs of the current device (cached per device; -1 if it cannot be asked)
+int cu_count() {
+  static std::atomic<int> cus[64];  // 0 = not asked yet (same answer from every thread)
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
   int n = cus[dev].load(std::memory_order_relaxed);
@@ -276,6 +276,13 @@ int launch_grid(int work_items) {
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return -1;
     cus[dev].store(n, std::memory_order_relaxed);
   }
+  return n;
+}
+
+// One persistent workgroup per CU (LDS allows no more), in multiples of the 8 XCDs.
+int launch_grid(int work_items) {
+  const int n = cu_count();
+  if (n <= 0) return -1;
   int g = (n / 8) * 8;
   if (g < 8) g = 8;
   return work_items < g ? work_items : g;
@@ -510,10 +517,15 @@ int run_bwd_keys(const intra::BParams& p, hipStream_t stream) {
 }
 
 // Queries per workgroup of the pass over the `ns` leading keys (LLM sinks, image text keys): about
-// one workgroup per CU, at least 128 queries each, a multiple of 64.
-int leading_chunk(int S, int B, int Hkv, int ns) {
+// one workgroup per CU (`cus`: the device's count; the workspace size and the launch have to use the
+// same one), at least 128 queries each, a multiple of 64.
+constexpr int MODEL_CUS = 256;  // host-only walks of the decomposition: any value gives a valid split
+// The workspace is sized for a device of WS_CUS CUs (no device has to be current to ask for the size);
+// a launch splits for min(its device's CUs, WS_CUS), which never needs more chunks than that.
+constexpr int WS_CUS = 320;
+int leading_chunk(int S, int B, int Hkv, int ns, int cus) {
   const int64_t row_wgs = (int64_t)B * Hkv * ((ns + 255) / 256);
-  int64_t chunks = std::max<int64_t>(1, 256 / row_wgs);  // at most one workgroup per CU: no second, thin round
+  int64_t chunks = std::max<int64_t>(1, cus / row_wgs);  // at most one workgroup per CU: no second, thin round
   chunks = std::min<int64_t>(chunks, std::max(1, S / 128));
   return (int)(64 * ((S + 64 * chunks - 1) / (64 * chunks)));
 }
@@ -550,11 +562,11 @@ int leading_keys(const Request& r) {
 
 // floats of workspace: D = rowsum(dO o O) per (batch, head, token), then the partial sums of the leading keys
 int64_t bwd_dsum_floats(int B, int S, int H) { return ((int64_t)B * H * S + 3) & ~(int64_t)3; }
-int64_t bwd_workspace_floats(const Request& r) {
+int64_t bwd_workspace_floats(const Request& r, int cus) {
   int64_t n = bwd_dsum_floats(r.B, r.S, r.H);
   const int ns = leading_keys(r);
   if (ns > 0) {
-    const int chunk = leading_chunk(r.S, r.B, r.Hkv, ns);
+    const int chunk = leading_chunk(r.S, r.B, r.Hkv, ns, cus);
     n += (int64_t)((r.S + chunk - 1) / chunk) * r.B * r.Hkv * ns * 128;
   }
   return n;
@@ -629,7 +641,9 @@ int run_bwd(int domain, const void* q, const void* k, const void* v, const void*
   const int ns = leading_keys(r);
   if (ns > 0) {
     p.geom.ns = ns;
-    p.geom.sink_chunk = leading_chunk(S, B, Hkv, ns);
+    const int cus = cu_count();
+    if (cus <= 0) return fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
+    p.geom.sink_chunk = leading_chunk(S, B, Hkv, ns, std::min(cus, WS_CUS));
   }
   hipStream_t st = static_cast<hipStream_t>(stream);
   switch (sh.map) {
@@ -721,7 +735,7 @@ int model_mask_bwd(const Request& r, uint8_t* count) {
     default: return fail(INTRA_ERR_UNSUPPORTED, "backward: no kernels for this pattern");
   }
   if (leading_keys(r) > 0) {
-    sh.geom.sink_chunk = leading_chunk(r.S, 1, 1, leading_keys(r));
+    sh.geom.sink_chunk = leading_chunk(r.S, 1, 1, leading_keys(r), MODEL_CUS);
     bwd_walk<intra::KeyRowsSinks>(sh.geom, count);
   }
   return INTRA_OK;
@@ -743,7 +757,7 @@ int model_mask_image_bwd(const Request& r, uint8_t* count) {
   if (!shape_for(r, 1, &sh)) return fail(INTRA_ERR_UNSUPPORTED, "no kernel shape for this request");
   IntraGeom ge = sh.geom;
   ge.ns = ge.text_len;  // the text keys are the leading keys every query sees
-  ge.sink_chunk = leading_chunk(r.S, 1, 1, ge.ns);
+  ge.sink_chunk = leading_chunk(r.S, 1, 1, ge.ns, MODEL_CUS);
   if (r.kind == KIND_IMG_SCATTER) {
     bwd_walk<intra::KeyRowsImgGroup<false>>(ge, count);
   } else {
@@ -815,7 +829,7 @@ int intra_llm_bwd_noalloc(const void* q, const void* k, const void* v, const voi
   int rc = make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true);
   if (rc) return rc;
   if ((rc = bwd_supported(r))) return rc;
-  const int64_t need = bwd_workspace_floats(r);
+  const int64_t need = bwd_workspace_floats(r, WS_CUS);
   if (need > (int64_t)INTRA_NOALLOC_SCRATCH_FLOATS)
     return fail(INTRA_ERR_UNSUPPORTED,
                 "intra_llm_bwd_noalloc: this call needs %lld floats of workspace, the built-in one holds %lld; "
@@ -833,7 +847,7 @@ int64_t intra_llm_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int g
   Request r;
   if (make_request(0, pattern, B, S, H, Hkv, group_num, window, &r, block, offset, n_sink, true)) return -1;
   if (bwd_supported(r)) return -1;
-  return bwd_workspace_floats(r);
+  return bwd_workspace_floats(r, WS_CUS);
 }
 
 int intra_image_bwd(const void* q, const void* k, const void* v, const void* o, const float* lse, const void* dout,
@@ -851,7 +865,7 @@ int64_t intra_image_bwd_workspace(int B, int S, int H, int Hkv, int pattern, int
   g_err[0] = 0;
   Request r;
   if (make_request(1, pattern, B, S, H, Hkv, width, text_len, &r)) return -1;
-  return bwd_workspace_floats(r);
+  return bwd_workspace_floats(r, WS_CUS);
 }
 
 int intra_model_mask_llm_bwd(int pattern, int S, int group_num, int window, int block, int offset, int n_sink,

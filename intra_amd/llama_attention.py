@@ -58,6 +58,10 @@ def intra_attention_forward(module, query, key, value, attention_mask=None, scal
         raise ValueError("the INTRA kernels need bfloat16 and head_dim 128")
     elif cfg["kind"] == "S":
         block = cfg.get("scatter_block", 1)
+        if block == 1 and not cfg.get("n_sink", 0):
+            # token-level Scatter (the reference's default scatter_blocks=(1,)): the plain Scatter kernel
+            out = _sparse("scatter", query, key, value, scaling, group_num=cfg["num_groups"])
+            return out.transpose(1, 2).contiguous(), None
         if block % 64:
             raise ValueError(f"block Scatter kernels need blocks of a multiple of 64 tokens (got {block})")
         if cfg.get("n_sink", 0) > block:
@@ -75,7 +79,7 @@ def _decoder_layers(model):
     return inner.layers
 
 
-def install_intra_llama(model, num_groups=8, window=512, dense_debug=False, n_sink=0, scatter_blocks=(256,),
+def install_intra_llama(model, num_groups=8, window=512, dense_debug=False, n_sink=0, scatter_blocks=(1,),
                         layer_pattern="SSWW", scatter_stripe=False, scatter_n_offsets=0):
     """Give every decoder layer its branch: the letters of `layer_pattern` ('S' Scatter, 'W' window,
     'D' dense) are cycled over the layers, `scatter_blocks` over the Scatter layers, and with
@@ -84,7 +88,7 @@ def install_intra_llama(model, num_groups=8, window=512, dense_debug=False, n_si
     choose between the reference's SDPA / FlexAttention code paths have no counterpart.  Returns
     the numbers of (Scatter, window, dense) layers."""
     layers = _decoder_layers(model)
-    blocks = list(scatter_blocks) or [256]
+    blocks = list(scatter_blocks) or [1]
     letters = [c for c in layer_pattern.upper() if c in "SWD"] or ["S", "S", "W", "W"]
     n_off = max(scatter_n_offsets, 0) or num_groups
     count = {"S": 0, "W": 0, "D": 0}

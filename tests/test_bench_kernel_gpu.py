@@ -50,8 +50,8 @@ def test_llm_rows(tmp_path):
         for key, (kind, kw) in kinds.items():
             flop = 4 * 128 * oracle.pairs_per_head(kind, S, **kw) * 32
             tf = flop / (r[key] * 1e-3) / 1e12
-            assert abs(r[key + "_tflops"] - tf) <= 0.06 + 1e-3 * tf, key      # rounded to 0.1; ms rounded to 1e-4
-            assert abs(r[key + "_pct_peak"] - 100 * tf / PEAK) <= 0.06 + 1e-3 * tf
+            assert abs(r[key + "_tflops"] - tf) <= 0.06 + 4e-3 * tf, key      # rounded to 0.1; ms (tens of us) rounded to 1e-4
+            assert abs(r[key + "_pct_peak"] - 100 * tf / PEAK) <= 0.06 + 4e-3 * tf
             assert r[key + "_cpu_ms"] > r[key]      # the fp32 dense-mask specification on the host cores
 
 
@@ -65,7 +65,7 @@ def test_image_rows(tmp_path):
     for key in ("scatter", "gather0"):
         flop = 4 * 128 * oracle.pairs_per_head("image/" + key, 4608, width=64) * 4
         tf = flop / (r[key] * 1e-3) / 1e12
-        assert abs(r[key + "_tflops"] - tf) <= 0.06 + 1e-3 * tf
+        assert abs(r[key + "_tflops"] - tf) <= 0.06 + 4e-3 * tf
         assert r[key + "_cpu_ms"] > r[key]
 
 

@@ -281,11 +281,12 @@ def test_bwd_validates_before_touching_the_gpu(lib):
     assert call(ptrs=(P,) * 9 + (P + 4,)) == _lib.INTRA_ERR_INVALID and "workspace" in _lib.last_error()
 
 
-def _leading_chunks(S, B, Hkv, ns):
-    """The library's rule for the pass over leading keys: about one workgroup per CU, chunks of at
-    least 128 queries and a multiple of 64."""
+def _leading_chunks(S, B, Hkv, ns, cus=320):
+    """The library's rule for the pass over leading keys: about one workgroup per CU (the workspace
+    is sized for a device of 320 CUs, whatever device is current), chunks of at least 128 queries and
+    a multiple of 64."""
     row_wgs = B * Hkv * -(-ns // 256)
-    chunks = min(max(1, 256 // row_wgs), max(1, S // 128))
+    chunks = min(max(1, cus // row_wgs), max(1, S // 128))
     chunk = 64 * -(-S // (64 * chunks))
     return -(-S // chunk)
 
@@ -294,9 +295,9 @@ def test_bwd_workspace_size(lib):
     assert lib.intra_llm_bwd_workspace(1, 1000, 8, 2, 0, 8, 576, 256, 0, 0) == 8000
     assert lib.intra_llm_bwd_workspace(2, 1001, 3, 3, 4, 8, 576, 256, 0, 0) == 6008  # rounded up to 4
     # sinks: chunks x B x Hkv x n_sink x 128 more
-    assert _leading_chunks(3000, 1, 2, 64) == 16 and _leading_chunks(65536, 1, 8, 64) == 32
+    assert _leading_chunks(3000, 1, 2, 64) == 16 and _leading_chunks(65536, 1, 8, 64) == 40
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 24000 + 16 * 2 * 64 * 128
-    assert lib.intra_llm_bwd_workspace(1, 65536, 32, 8, 9, 2, 575, 256, 0, 64) == 65536 * 32 + 32 * 8 * 64 * 128
+    assert lib.intra_llm_bwd_workspace(1, 65536, 32, 8, 9, 2, 575, 256, 0, 64) == 65536 * 32 + 40 * 8 * 64 * 128
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 256, 1, 0) == 24000
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 128, 1, 0) == -1
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 3, 0, 8, 576, 256, 0, 0) == -1

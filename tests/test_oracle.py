@@ -25,6 +25,27 @@ def test_llm_scatter_bruteforce(S, G):
             assert bool(m[a, b]) == (b <= a and a % G == b % G)
 
 
+@pytest.mark.parametrize("S,G", [(257, 8), (100, 3), (64, 2), (9, 16), (40, 1)])
+def test_llm_scatter_by_dealing(S, G):
+    # built from the prose, without the predicate: deal the tokens round-robin into G piles, in
+    # order; a token attends to the tokens that lie below it in its own pile and to itself.  Row
+    # counts follow: token i has i // G tokens below it.
+    piles = [[] for _ in range(G)]
+    want = torch.zeros(S, S, dtype=torch.bool)
+    for token in range(S):
+        pile = piles[token % len(piles)]
+        pile.append(token)
+        want[token, pile] = True
+    m = masks.llm_scatter_mask(S, G)
+    assert torch.equal(m, want)
+    assert m.sum(1).tolist() == [i // G + 1 for i in range(S)]
+    assert not bool(torch.triu(m, 1).any())                       # causal
+    assert int(m.sum()) == sum(len(p) * (len(p) + 1) // 2 for p in piles)
+    # Gather 1 with segments of one token is the same dealing
+    if G > 1:
+        assert torch.equal(masks.llm_block_scatter_mask(S, G, 1, 0, 0), want)
+
+
 @pytest.mark.parametrize("S,G", [(32, 4), (128, 8), (64, 8), (70, 3), (200, 8)])
 def test_llm_gather1_bruteforce(S, G):
     m = masks.llm_gather1_mask(S, G)

@@ -329,7 +329,7 @@ def test_calls_can_be_captured_in_a_graph_and_replayed():
     q, k, v = make_qkv(1, 4608, 8, 8, seed=41)
     calls = [lambda q, k, v: intra_llm_attn(q, k, v, "scatter", group_num=8),
              lambda q, k, v: intra_llm_attn(q, k, v, "window_sink", window=575, n_sink=64),
-             lambda q, k, v: intra_image_attn(q, k, v, "gather0", 64)]  # two launches
+             lambda q, k, v: intra_image_attn(q, k, v, "gather0", 64)]  # two kinds of sets in one launch
     with torch.no_grad():
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
