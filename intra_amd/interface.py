@@ -49,22 +49,28 @@ def get_softmax_mode():
     return {v: k for k, v in SOFTMAX_MODES.items()}[_C.intra_get_softmax_mode()]
 
 
+_BF16 = torch.bfloat16
+
+
 def _check(q, k, v, forward_call=True):
-    # reference: intra_attn/interface.py:17-23 (same conditions, same exception types and texts)
-    for x in (q, k, v):
-        if not x.is_cuda or x.dtype != torch.bfloat16 or x.shape[-1] != 128:
-            raise ValueError("INTRA kernels need CUDA bfloat16 tensors with head_dim 128")
+    # reference: intra_attn/interface.py:17-23 (same conditions, same exception types and texts);
+    # written flat because this runs in front of kernels that take a few tens of microseconds
+    qs, ks, vs = q.shape, k.shape, v.shape
+    if not (q.is_cuda and k.is_cuda and v.is_cuda and q.dtype is _BF16 and k.dtype is _BF16 and v.dtype is _BF16
+            and qs[-1] == 128 and ks[-1] == 128 and vs[-1] == 128):
+        raise ValueError("INTRA kernels need CUDA bfloat16 tensors with head_dim 128")
     # the plain forward calls record no graph (intra_llm_attn_func / intra_image_attn_func do)
-    if forward_call and torch.is_grad_enabled() and any(x.requires_grad for x in (q, k, v)):
+    if forward_call and (q.requires_grad or k.requires_grad or v.requires_grad) and torch.is_grad_enabled():
         raise RuntimeError("INTRA kernels are forward-only; call them under torch.no_grad()")
-    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+    if len(qs) != 4 or len(ks) != 4 or len(vs) != 4:
         raise ValueError("q, k, v must be (batch, seqlen, heads, 128)")
-    if k.shape != v.shape or k.shape[:2] != q.shape[:2] or q.shape[2] % k.shape[2]:
-        raise RuntimeError(f"q {tuple(q.shape)} and k/v {tuple(k.shape)}/{tuple(v.shape)} do not "
+    if ks != vs or ks[0] != qs[0] or ks[1] != qs[1] or qs[2] % ks[2]:
+        raise RuntimeError(f"q {tuple(qs)} and k/v {tuple(ks)}/{tuple(vs)} do not "
                            "match: need equal batch and seqlen, and query heads divisible by kv heads")
     # The kernels honour arbitrary batch/token/head strides; only rows that are not contiguous
     # or not 16-byte aligned are copied.
-    return [x if _aligned(x) else x.contiguous() for x in (q, k, v)]
+    return (q if _aligned(q) else q.contiguous(), k if _aligned(k) else k.contiguous(),
+            v if _aligned(v) else v.contiguous())
 
 
 def _scale(q, softmax_scale):
