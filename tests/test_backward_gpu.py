@@ -12,7 +12,10 @@ The kernels round the softmax weights and their derivatives to bf16 before the s
 D = dout . out from the bf16 output, and round the results to bf16 (2^-9).  The terms that add up
 to one gradient element partly cancel, so an element's error scales with the tensor, not with the
 element: hence the m / 64.  The norm bound is the sharp one: a dropped term, a wrong scale or a
-missed key block moves it by orders of magnitude."""
+missed key block moves it by orders of magnitude.
+Observed over all comparisons of this file, test_backward_image_gpu.py and test_llama_caller_gpu.py
+(477 tensors): the worst element is at (m + |want|) / 169, the worst tensor at ||want||_2 / 212, so
+the two bounds sit at 2.6 and 1.7 times what occurs."""
 import pytest
 import torch
 
