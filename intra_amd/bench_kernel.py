@@ -15,8 +15,9 @@ build of the library (python -m intra_amd.build --diag), selected through INTRA_
     INTRA_HIP_LIB=intra_amd/libintra_hip_diag.so python -m intra_amd.bench_kernel phases \
         --pattern scatter --seqlen 32768 [--softmax exact]
 
-`ceiling`: what the matrix cores sustain with nothing else running, with constant and with random
-operand bits, and the clock they run at (the board is power-limited):
+`ceiling`: what the matrix cores sustain with nothing else running, per MFMA shape (16x16x32 and
+32x32x16), with constant and with random operand bits, and the clock they run at (the board is
+power-limited):
 
     python -m intra_amd.bench_kernel ceiling
 """
@@ -286,8 +287,9 @@ def bench_phases(args):
 
 
 def bench_ceiling(args):
-    """MFMA-only launch (8 wavefronts per CU on every CU, nothing but v_mfma_f32_32x32x16_bf16) with
-    constant and with random operand bits: TFLOP/s and the shader clock it ran at."""
+    """MFMA-only launches (8 wavefronts per CU on every CU, nothing but v_mfma_f32_16x16x32_bf16, the
+    forward kernel's instruction, or v_mfma_f32_32x32x16_bf16, the backward kernels') with constant
+    and with random operand bits: TFLOP/s and the shader clock each ran at."""
     lib = _lib.load()
     n_wg = torch.cuda.get_device_properties(0).multi_processor_count
     iters = 20000
@@ -297,20 +299,20 @@ def bench_ceiling(args):
     tables = {"constant 1.0": torch.full((65536,), 1.0).to(torch.bfloat16),
               "random N(0,1)": torch.randn(65536, generator=g).to(torch.bfloat16)}
     rows = []
-    for name, host in tables.items():
+    for shape, name, host in [(sh, n, h) for sh in (16, 32) for n, h in tables.items()]:
         table = host.cuda()
         stream = torch.cuda.current_stream().cuda_stream
         best = None
         for rep in range(4):
             tic, toc = (torch.cuda.Event(enable_timing=True) for _ in range(2))
             tic.record()
-            rc = lib.intra_diag_mfma_ceiling(table.data_ptr(), sink.data_ptr(), clocks.data_ptr(), n_wg, iters, stream)
+            rc = lib.intra_diag_mfma_ceiling(table.data_ptr(), sink.data_ptr(), clocks.data_ptr(), n_wg, iters, shape, stream)
             assert rc == 0, _lib.last_error()
             toc.record()
             toc.synchronize()
             ms = tic.elapsed_time(toc)
             c = clocks.view(-1, 2).double().cpu()
-            row = {"operands": name, "workgroups": n_wg, "ms": round(ms, 3),
+            row = {"mfma": "16x16x32" if shape == 16 else "32x32x16", "operands": name, "workgroups": n_wg, "ms": round(ms, 3),
                    "tflops": round(n_wg * 8 * iters * 16 * 32768 / (ms * 1e-3) / 1e12, 1),
                    "shader_clock_mhz": round((c[:, 0] / c[:, 1]).mean().item() * 100, 1)}
             if rep > 0 and (best is None or row["ms"] < best["ms"]):  # first launch: clock still ramping

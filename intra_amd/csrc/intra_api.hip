@@ -917,14 +917,19 @@ int intra_diag_set_buffer(long long* counters, int64_t n_values) {
 }
 
 int intra_diag_mfma_ceiling(const void* table, float* sink, long long* clocks, int workgroups, int iters,
-                            void* hip_stream) {
+                            int shape, void* hip_stream) {
   g_err[0] = 0;
   if (!table || !sink || !clocks) return fail(INTRA_ERR_INVALID, "table, sink and clocks must be non-null device pointers");
   if (!aligned16(table)) return fail(INTRA_ERR_INVALID, "table must be 16-byte aligned");
   if (workgroups < 1 || workgroups > 65536 || iters < 1)
     return fail(INTRA_ERR_INVALID, "workgroups must be in [1, 65536] and iters positive (got %d, %d)", workgroups, iters);
-  hipLaunchKernelGGL(intra::mfma_ceiling_kernel, dim3(workgroups), dim3(512), 0, static_cast<hipStream_t>(hip_stream),
-                     static_cast<const uint4*>(table), sink, iters, clocks);
+  if (shape != 16 && shape != 32) return fail(INTRA_ERR_INVALID, "shape must be 16 (16x16x32) or 32 (32x32x16), got %d", shape);
+  if (shape == 16)
+    hipLaunchKernelGGL(intra::mfma_ceiling_kernel<true>, dim3(workgroups), dim3(512), 0, static_cast<hipStream_t>(hip_stream),
+                       static_cast<const uint4*>(table), sink, iters, clocks);
+  else
+    hipLaunchKernelGGL(intra::mfma_ceiling_kernel<false>, dim3(workgroups), dim3(512), 0, static_cast<hipStream_t>(hip_stream),
+                       static_cast<const uint4*>(table), sink, iters, clocks);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
   return INTRA_OK;

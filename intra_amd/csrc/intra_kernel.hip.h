@@ -7,16 +7,20 @@
 //  * A workgroup of NW wavefronts owns a row block of one set: POS = NW*32/HP consecutive in-set
 //    queries of HP query heads that share one KV head (GQA packing), so every gathered K/V tile
 //    is used by all HP heads.  Each wavefront owns 32 queries of one head.
-//  * Scores are computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: the A operand
-//    is a K tile row read from LDS (16 B per lane), the B operand is Q held in registers for the
-//    whole kernel.  In the accumulator layout a lane then holds 16 keys of ONE query per 32x32
-//    block, so the online softmax needs a single cross-lane exchange (lane ^ 32) per tile and the
-//    rescale factors are plain per-lane scalars.
+//  * Scores are computed transposed, S^T = K Q^T, with v_mfma_f32_16x16x32_bf16 (per flop it draws
+//    about a tenth less power than the 32x32x16 shape, and this kernel runs against the board's
+//    power limit): the A operand is a K tile row read from LDS (16 B per lane), the B operand is Q
+//    held in registers for a whole work item.  A 32-key block times the wavefront's 32 queries is
+//    2 x 2 tiles; in the accumulator layout a lane holds 4 keys per tile of ONE query per query
+//    tile, so the rescale factors are plain per-lane scalars and a query's maximum or sum is a
+//    reduction over four lanes (l, l ^ 16, l ^ 32, l ^ 48).
 //  * O^T = V^T P^T: P^T is the softmax output still in registers (packed to bf16, no LDS round
-//    trip); V^T comes from ds_read_b64_tr_b16 transposing reads of the row-major V tile.
-//  * Software pipeline in steps of 32 keys: in step j a wavefront issues the 8 QK^T MFMAs of key
-//    block j+1 and the 8 PV MFMAs of block j, with the softmax VALU work of block j spread over
-//    both phases and every LDS operand read issued a whole phase (8 MFMAs) ahead.
+//    trip): the lane's 8 weights of a query tile ARE its B operand, under a numbering of the 32-key
+//    reduction that the V^T operand follows; V^T comes from ds_read_b64_tr_b16 transposing reads of
+//    the row-major V tile.
+//  * Software pipeline in steps of 32 keys: in step j a wavefront issues the 16 QK^T MFMAs of key
+//    block j+1 and the 16 PV MFMAs of block j, with the softmax VALU work of block j spread over
+//    both phases and every LDS operand read issued about a phase ahead.
 //  * K/V rows are gathered from HBM straight into LDS (global_load_lds_dwordx4, 16 lanes per
 //    256-byte row, no register staging), three tiles ahead; one barrier per 64-key tile, which
 //    only waits for the requests of the previous iteration.  The tiles of all work items of a
@@ -25,9 +29,10 @@
 //    two ring slots in front of its key tiles: they are requested three slots ahead like any
 //    tile, arrive as whole 256-byte rows, and each wavefront picks its 32 rows out of LDS with
 //    the K operand's read pattern.  The output rows of a finished item stay in registers until
-//    the next item's first requests are out and are stored behind them.  An LDS tile is 16 groups of 4 rows with an XOR chunk
-//    swizzle inside the group and 16 bytes of padding between groups, so the row-per-lane K reads
-//    and the 4-row transposing V reads are both free of bank conflicts.
+//    the next item's first requests are out and are stored behind them.  An LDS tile is 16 groups
+//    of 4 rows with an XOR chunk swizzle inside the group and padding between groups (16 bytes in K
+//    tiles, 32 in V tiles), so the row-per-lane K reads and the 4-row transposing V reads are both
+//    free of bank conflicts.
 //  * The softmax reference stays 0 (weights exp2(score*c), exact after normalisation because
 //    numerator and denominator share it) unless a block maximum leaves the +-60 exponent band;
 //    then the query is re-centred and O rescaled.  No per-block rescale in the common case.
@@ -56,6 +61,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef float floatx2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -112,18 +118,23 @@ constexpr int BN = 64;             // keys per tile (one barrier per tile)
 // LDS tile layout.  A tile is 16 groups of 4 rows; a group is 1024 contiguous bytes (what one
 // 16-bytes-per-lane direct-to-LDS load instruction writes) followed by 16 bytes of padding.
 // Inside a group, the 16-byte chunk c of row i (0..3) sits at chunk slot c ^ (4 * i).  With
-// that, 16 consecutive rows read at one chunk (the K operand pattern) and the 4 rows x 64 bytes
-// of a transposing V read both touch 16 distinct 16-byte bank groups.
+// that, 16 consecutive rows read at one chunk (the K operand pattern) touch 16 distinct 16-byte
+// bank groups (and so do the 4 rows x 64 bytes of the backward kernels' transposing reads).
 constexpr int GROUP_STRIDE = 1024 + 16;
 constexpr int TILE_BYTES = (BN / 4) * GROUP_STRIDE;
+// The V tiles of the forward kernel pad their groups by 32 bytes instead: its transposing reads
+// take the 4 rows x 32 bytes of TWO neighbouring groups per half wavefront, and the two groups
+// must not share a 16-byte bank group.
+constexpr int VGROUP_STRIDE = 1024 + 32;
 constexpr int KTILE = TILE_BYTES;
-constexpr int VTILE = TILE_BYTES;
+constexpr int VTILE = (BN / 4) * VGROUP_STRIDE;
 constexpr int NKBUF = 4, NVBUF = 4;   // tiles i-1 (being overwritten) .. i+2 of K and of V
 constexpr int VBASE = NKBUF * KTILE;  // K ring then V ring
 constexpr int RING_BYTES = NKBUF * KTILE + NVBUF * VTILE;
 constexpr int REDO_WORDS = 64;        // bitmap of work-item rounds to run again in EXACT mode (round % 2048)
 constexpr int LDS_BYTES = RING_BYTES + REDO_WORDS * 4;
-constexpr int BLOCK32 = 8 * GROUP_STRIDE;  // 32 rows
+constexpr int BLOCK32 = 8 * GROUP_STRIDE;    // 32 rows
+constexpr int VBLOCK32 = 8 * VGROUP_STRIDE;  // 32 rows of a forward V tile
 
 // 64 lanes x 16 bytes from per-lane global addresses to 1024 consecutive LDS bytes at lds_addr
 // (wave-uniform).  Issued as inline assembly so that the compiler does not put a full vmcnt(0)
@@ -152,6 +163,16 @@ __device__ __forceinline__ float lane_xor32_sum(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
+// the same over the four lanes l % 16, l % 16 + 16, + 32, + 48 (the lanes that share a query in the
+// 16x16 accumulator layout of the forward kernel)
+__device__ __forceinline__ float lane_quad_max(float x) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return lane_xor32_max(fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1])));
+}
+__device__ __forceinline__ float lane_quad_sum(float x) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return lane_xor32_sum(__uint_as_float(r[0]) + __uint_as_float(r[1]));
+}
 
 template <int V>
 using ic = std::integral_constant<int, V>;
@@ -167,8 +188,8 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int h32 = lane >> 5;  // which half of the wavefront
-  const int l32 = lane & 31;
+  const int l16 = lane & 15;  // row or column of a 16x16 MFMA tile
+  const int g4 = lane >> 4;   // which quarter of the wavefront
 
   // ---------------------------------------------------------------- persistent loop over work items
   // The grid holds about one workgroup per CU and every workgroup walks through several work items
@@ -263,7 +284,8 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   if (!locate(0, cw)) return;
   INTRA_DIAG(long long dg[DIAG_SLOTS] = {0, 0, 0, 0, 0, 0, 0, 0};)
   Feed fd = feed_for(cw, -1);
-  auto feed_tile = [&](int slot_off) {  // request the next slot of the stream into a ring slot
+  // request the next slot of the stream into a ring slot (byte offsets inside the K and V rings)
+  auto feed_tile = [&](int koff, int voff) {
     if (fd.tile < 0) {  // 128 Q rows: rows of four wavefronts, two per part
 #pragma unroll
       for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
@@ -275,7 +297,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
           const int t = im_min(fd.t0 + (wq / HP) * 32 + (rho & 31), fd.t1);
           const uint32_t pos = fd.map.qpos(t);
           dma_group(fd.qbase + ((int64_t)(wq % HP) * p.q_hs * 2 + (uint64_t)pos * q_rs_b + ld_col),
-                    lds_base + part * VBASE + slot_off + grp * GROUP_STRIDE);
+                    lds_base + (part ? VBASE + voff + grp * VGROUP_STRIDE : koff + grp * GROUP_STRIDE));
         }
       }
     } else {
@@ -284,8 +306,8 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
         const int grp = wave * GROUPS_PER_WAVE + gi;
         const int tk = im_min(fd.rg.kt_lo + fd.tile * BN + 4 * grp + ld_row, fd.nk - 1);
         const uint32_t pos = fd.map.kpos(tk);
-        dma_group(fd.kbase + ((uint64_t)pos * k_rs_b + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
-        dma_group(fd.vbase + ((uint64_t)pos * v_rs_b + ld_col), lds_base + VBASE + slot_off + grp * GROUP_STRIDE);
+        dma_group(fd.kbase + ((uint64_t)pos * k_rs_b + ld_col), lds_base + koff + grp * GROUP_STRIDE);
+        dma_group(fd.vbase + ((uint64_t)pos * v_rs_b + ld_col), lds_base + VBASE + voff + grp * VGROUP_STRIDE);
       }
     }
     ++fd.tile;
@@ -297,63 +319,53 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   };
   constexpr int PER_TILE = 2 * GROUPS_PER_WAVE;  // requests per wavefront per slot (K + V parts)
 
-  // LDS operand addresses.  With the chunk swizzle c ^ 4i of a group, the 16-byte chunk 2*ks + h32
-  // of key row l32 (the K operand of k-step ks = 2a + b) sits at byte 64 * (a ^ r) + 32 * b +
-  // 16 * h32 of its row slot, r = l32 % 4: four lane-dependent bases (one per a) and compile-time
-  // offsets for everything else, which the ds_read offset field takes.  The bases carry the ring
-  // slot and are advanced once per tile: kb[] follows the tile AFTER the one being multiplied
-  // (whose K rows the pipeline reads ahead), vb[] the current one.
+  // LDS operand addresses.  A 32-key block times the wavefront's 32 queries is 2 x 2 MFMA tiles of
+  // 16 x 16 with 4 k-steps of 32 head dims; lane (l16, g4) supplies head dims 32 * ks + 8 * g4 .. + 7,
+  // the 16-byte chunk 4 * ks + g4, of key row 16 * kt + l16.  With the chunk swizzle c ^ 4i of a
+  // group that chunk sits at byte 64 * (ks ^ r) + 16 * g4 of its row slot, r = l16 % 4: four
+  // lane-dependent bases (one per ks) and compile-time offsets for everything else, which the
+  // ds_read offset field takes.  The bases carry the ring slot and are advanced once per tile:
+  // kb[] follows the tile AFTER the one being multiplied (whose K rows the pipeline reads ahead),
+  // vb[] the current one.
+  const int lane_chunks = (l16 & 3) * 256 + 16 * g4;  // row slot inside the group + chunk g4, before the swizzle
   int kb[4], vb[4];
   {
-    const int r = l32 & 3;
+    const int r = l16 & 3;
 #pragma unroll
-    for (int a = 0; a < 4; ++a) kb[a] = KTILE + (l32 >> 2) * GROUP_STRIDE + r * 256 + 64 * (a ^ r) + 16 * h32;
+    for (int ks = 0; ks < 4; ++ks) kb[ks] = KTILE + (l16 >> 2) * GROUP_STRIDE + lane_chunks + 64 * (ks ^ r);
     // V^T operand (A of O^T = V^T P^T) through transposing reads.  Within each group of 16 lanes,
     // lane i supplies the address of 4 head dims (4*(i%4)..) of key row i/4 and receives head dim i
-    // of those 4 key rows.  Lane groups 0/1 take head dims 0-15/16-31 of a 32-dim block, the upper
-    // 32 lanes the key rows 4..7 of each 8 (the next 4-row group).  vb[db]: 32-dim block db.
-    const int i16 = lane & 15, g2 = (lane >> 4) & 1, ri = i16 >> 2;
+    // of those 4 key rows.  The MFMA's 32-key reduction is numbered so that lane quarter g4 holds
+    // keys 4*g4 .. +3 and 16 + 4*g4 .. +3 of the block (what the score accumulators of that lane
+    // hold, see below): two reads, of row groups g4 and 4 + g4.  vb[a]: head dims 32*a .. 32*a+31,
+    // the 16-dim tile 2*a + b another 32 bytes further.
+    const int ri = l16 >> 2;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
-      vb[db] = VBASE + h32 * GROUP_STRIDE + ri * 256 + 64 * (db ^ ri) + 16 * (2 * g2 + ((i16 & 3) >> 1)) + 8 * (i16 & 1);
+    for (int a = 0; a < 4; ++a)
+      vb[a] = VBASE + g4 * VGROUP_STRIDE + ri * 256 + 64 * (a ^ ri) + 16 * ((l16 & 3) >> 1) + 8 * (l16 & 1);
   }
-  // Q^T fragments: lane holds query l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
-  bf16x8 qf[8];
-  auto kread_q = [&](int base, int off) { return *reinterpret_cast<const bf16x8*>(smem + (base + off)); };
-  // O is stored 64 contiguous bytes per row and instruction instead of 32: the two lanes of
-  // neighbouring queries 2a, 2a+1 (and their upper-half twins) together cover chunks 4m..4m+3 of
-  // row 2a in access 2m and of row 2a+1 in access 2m+1, lane (e = query parity, h) taking chunk
-  // 4m + 2e + h.  A lane holds its own chunks 2ks + h for every ks; those with ks != e (mod 2) are
-  // swapped with its neighbour's, one quad permute per dword (pair_exchange).
-  const int qpar = l32 & 1;
-  auto pair_exchange = [&](u32x4 (&r)[8]) {
-#pragma unroll
-    for (int m = 0; m < 4; ++m)
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        const uint32_t x0 = r[2 * m][d], x1 = r[2 * m + 1][d];
-        const uint32_t got = (uint32_t)__builtin_amdgcn_mov_dpp((int)(qpar ? x0 : x1), 0xB1, 0xF, 0xF, true);  // lane ^ 1
-        r[2 * m][d] = qpar ? got : x0;
-        r[2 * m + 1][d] = qpar ? x1 : got;
-      }
-  };
+  // Q^T fragments (B operand of S^T = K Q^T): qf[qt][ks] is chunk 4 * ks + g4 of query 16 * qt + l16
+  bf16x8 qf[2][4];
+  auto kread_q = [&](int addr) { return *reinterpret_cast<const bf16x8*>(smem + addr); };
 
-  // Ring slots (byte offsets into the K ring; the V ring uses the same offsets behind VBASE) of
-  // the stream tiles i, i+1, i+2, i+3 seen from the computation; they rotate once per tile and
-  // carry on from one work item to the next.
+  // Ring slots (byte offsets into the K ring and into the V ring) of the stream tiles i, i+1, i+2,
+  // i+3 seen from the computation; they rotate once per tile and carry on from one work item to
+  // the next.
   int k0 = 0, k1 = KTILE, k2 = 2 * KTILE, k3 = 3 * KTILE;
-  feed_tile(k0);  // the two Q slots of the first work item and its first key tile
-  feed_tile(k1);
-  feed_tile(k2);
+  int v0 = 0, v1 = VTILE, v2 = 2 * VTILE, v3 = 3 * VTILE;
+  feed_tile(k0, v0);  // the two Q slots of the first work item and its first key tile
+  feed_tile(k1, v1);
+  feed_tile(k2, v2);
   auto rotate = [&] {  // one slot further in the stream
-    const int dk = k2 - k1, dv = k1 - k0;  // +KTILE, or -3 * KTILE where the ring wraps
+    const int dk = k2 - k1, dv = v1 - v0;  // one tile, or minus three where the ring wraps
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       kb[a] += dk;
       vb[a] += dv;
     }
-    const int tk = k0;
+    const int tk = k0, tv = v0;
     k0 = k1; k1 = k2; k2 = k3; k3 = tk;
+    v0 = v1; v1 = v2; v2 = v3; v3 = tv;
   };
   // Barrier in front of a slot, leaving this wavefront's requests for the slot after the next in
   // flight (the PER_TILE most recent operations) and, where they were issued in between, the
@@ -364,16 +376,18 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     else if (extra == 8) tile_barrier<PER_TILE + 8>();
     else tile_barrier<PER_TILE + 9>();
   };
-  // Output of the finished work item, kept in registers until the next item's first requests are out
+  // Output of the finished work item, kept in registers until the next item's first requests are
+  // out: pk[4 * qt + m] is the 16-byte chunk 4 * m + 2 * (g4 % 2) + g4 / 2 of the row of query qt,
+  // so the four lanes of a query store 64 contiguous bytes per instruction.
   u32x4 pk[8];
-  uint16_t *orow_a = nullptr, *orow_b = nullptr;
+  uint16_t* orow[2] = {nullptr, nullptr};
   float* lse_dst = nullptr;
   float lse_val = 0.f;
   int held = 0;  // vector-memory operations the held output will take: 0 (nothing held), 8, or 9 with a log-sum-exp
   auto store_held = [&] {
     if (held == 0) return;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(((i & 1) ? orow_b : orow_a) + 32 * (i >> 1)) = pk[i];
+    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(orow[i >> 2] + 32 * (i & 3)) = pk[i];
     if (held == 9) *lse_dst = lse_val;
   };
 
@@ -390,14 +404,25 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   const int kt_lo = rg.kt_lo, ntiles = rg.ntiles;
 
   // ---------------------------------------------------------------- this wavefront's queries
+  // A lane works for two queries: 16 * qt + l16 of the wavefront's 32, qt = 0, 1.  Rows past the
+  // end of the row block are clamped to its last row, for Q and for O alike: such lanes compute
+  // that row once more and store the same bytes to the same place, so every active wavefront
+  // issues all of its stores.
   const int hw = wave % HP;
   const int wq0 = t0 + (wave / HP) * 32;
   const bool wave_active = wq0 <= t1;
   const int wq_last = im_min(wq0 + 31, t1);
-  const bool row_valid = wq0 + l32 <= t1;
-  const int tq = im_min(wq0 + l32, t1);
-  const int lo_l = map.klo(tq);
-  const int hi_l = im_min(map.khi(tq), nk - 1);
+  bool row_valid[2];
+  int lo_l[2], hi_l[2];
+  int64_t qpos[2];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    row_valid[qt] = wq0 + 16 * qt + l16 <= t1;
+    const int tq = im_min(wq0 + 16 * qt + l16, t1);
+    lo_l[qt] = map.klo(tq);
+    hi_l[qt] = im_min(map.khi(tq), nk - 1);
+    qpos[qt] = map.qpos(tq);
+  }
   WaveBounds wb = wave_bounds(map, im_min(wq0, t1), wq_last);
   // 32-key blocks (counted from kt_lo) this wavefront has to look at: those of its own key range
   // and, for maps with a prefix, the prefix blocks in front of it.
@@ -416,130 +441,140 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   wb.w_hi = __builtin_amdgcn_readfirstlane(wb.w_hi);
 
   const int hq = kvh * p.ratio + hg * HP + hw;
-  const int64_t qpos = map.qpos(tq);
-  // The two rows this lane stores parts of.  Rows past the end of the row block are clamped to its
-  // last row, for Q and for O alike: such lanes compute that row once more and store the same
-  // bytes to the same place, so every active wavefront issues all of its stores.
-  const int ra = wq0 + (l32 & ~1);
-  const int64_t opos_a = map.qpos(im_min(ra, t1)), opos_b = map.qpos(im_min(ra + 1, t1));
 
   // ---------------------------------------------------------------- slot -2: the Q rows arrive
   INTRA_DIAG(const long long t_b = wall_clock64();)
   tile_barrier<PER_TILE>();  // both Q slots have landed; the held stores are not out yet
   INTRA_DIAG(const long long t_c = wall_clock64();)
-  feed_tile(k3);
+  feed_tile(k3, v3);
   store_held();              // behind the request, so that two more barriers can leave them in flight
   const int in_flight = held;
   held = 0;
   {
-    // this wavefront's 32 rows: slot wave / 4 (k0 or k1), part (wave / 2) % 2, rows 32 * (wave % 2) ..
-    const int qoff = ((wave >> 2) ? 0 : k0 - k1) + ((wave >> 1) & 1) * VBASE + (wave & 1) * BLOCK32;
+    // this wavefront's 32 rows: slot wave / 4 (ring slot 0 or 1 of the stream as it stands), part
+    // (wave / 2) % 2, rows 32 * (wave % 2) .. of the part; read with the K operand's pattern
+    int qa, qstep;  // address of row l16's chunk g4 before the k-step swizzle; bytes from query tile 0 to 1
+    if ((wave >> 1) & 1) {
+      qa = VBASE + ((wave >> 2) ? v1 : v0) + (wave & 1) * VBLOCK32 + (l16 >> 2) * VGROUP_STRIDE + lane_chunks;
+      qstep = 4 * VGROUP_STRIDE;
+    } else {
+      qa = ((wave >> 2) ? k1 : k0) + (wave & 1) * BLOCK32 + (l16 >> 2) * GROUP_STRIDE + lane_chunks;
+      qstep = 4 * GROUP_STRIDE;
+    }
+    const int r = l16 & 3;
     u32x4 raw[8];
 #pragma unroll
-    for (int g = 0; g < 8; ++g) raw[g] = __builtin_bit_cast(u32x4, kread_q(kb[g >> 1] + qoff, 32 * (g & 1)));
+    for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) raw[4 * qt + ks] = __builtin_bit_cast(u32x4, kread_q(qa + qt * qstep + 64 * (ks ^ r)));
     if (FAST) {  // Q <- bf16(Q * softmax_scale * log2 e): the MFMA then yields exponents directly
       const float cq = p.q_fold;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks)
+      for (int f = 0; f < 8; ++f)
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const uint32_t x = raw[ks][d];
-          floatx2 f = {__uint_as_float(x << 16) * cq, __uint_as_float(x & 0xffff0000u) * cq};
-          raw[ks][d] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+          const uint32_t x = raw[f][d];
+          floatx2 y = {__uint_as_float(x << 16) * cq, __uint_as_float(x & 0xffff0000u) * cq};
+          raw[f][d] = __builtin_bit_cast(uint32_t, __builtin_convertvector(y, bf16x2));
         }
+    } else if (p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
+#pragma unroll
+      for (int f = 0; f < 8; ++f) raw[f] ^= 0x80008000u;
     }
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[ks] = __builtin_bit_cast(bf16x8, raw[ks]);
+    for (int f = 0; f < 8; ++f) qf[f >> 2][f & 3] = __builtin_bit_cast(bf16x8, raw[f]);
   }
   rotate();
-  if (!FAST && p.negate_q) {  // softmax_scale < 0: flip the sign of Q (exact) and use |scale| below
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
-      qf[ks] = __builtin_bit_cast(bf16x8, __builtin_bit_cast(u32x4, qf[ks]) ^ 0x80008000u);
-  }
 
   // ---------------------------------------------------------------- running softmax state
-  floatx16 oacc[4];
+  // oacc[dt][qt]: O^T tile of head dims 16 * dt .. + 15 and query tile qt; the lane holds head dims
+  // 16 * dt + 4 * g4 .. + 3 of query 16 * qt + l16.
+  floatx4 oacc[8][2];
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) oacc[db][e] = 0.f;
-  floatx16 s0, s1;  // raw scores q.k of two consecutive 32-key blocks
-  // Exponent reference of this lane's query.  Weights are exp2(score * c - mref) and numerator and
-  // denominator always share mref, so any value gives the exact softmax as long as nothing
-  // overflows or underflows.  fp32 and bf16 both span 2^+-126, so mref stays 0 (and costs nothing)
-  // for every query whose scores stay within +-60 of it; it is re-centred on a block's maximum
-  // when that maximum leaves this band upwards, or downwards before anything was accumulated.
-  // FAST mode has no reference at all (weights exp2(score), scores already in exponent units).
-  float mref = 0.f;
-  float l_acc[2] = {0.f, 0.f};  // two partial row sums of the weights (summed at the end)
+    for (int qt = 0; qt < 2; ++qt) oacc[dt][qt] = floatx4{0.f, 0.f, 0.f, 0.f};
+  // Raw scores q.k of two consecutive 32-key blocks, [kt][qt]: the lane holds keys
+  // 16 * kt + 4 * g4 .. + 3 of the block for query 16 * qt + l16.
+  floatx4 s0[2][2], s1[2][2];
+  // Exponent reference of each of the lane's queries.  Weights are exp2(score * c - mref) and
+  // numerator and denominator always share mref, so any value gives the exact softmax as long as
+  // nothing overflows or underflows.  fp32 and bf16 both span 2^+-126, so mref stays 0 (and costs
+  // nothing) for every query whose scores stay within +-60 of it; it is re-centred on a block's
+  // maximum when that maximum leaves this band upwards, or downwards before anything was
+  // accumulated.  FAST mode has no reference at all (weights exp2(score), scores already in
+  // exponent units).
+  float mref[2] = {0.f, 0.f};
+  float l_acc[2] = {0.f, 0.f};  // this lane's share of the two queries' weight sums
   const float c = p.scale_log2;  // |softmax_scale| * log2(e)
   const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
   // operand reads: base register + compile-time byte offset
   auto kread_at = [&](int base, int off) { return *reinterpret_cast<const bf16x8*>(smem + (base + off)); };
   auto vread_at = [&](int base, int off) {
-    bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(smem + (base + off)));
-    bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (__attribute__((address_space(3))) bf16x4*)(smem + (base + off + 2 * GROUP_STRIDE)));
-    return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+    bf16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(smem + (base + off)));
+    bf16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (__attribute__((address_space(3))) bf16x4*)(smem + (base + off + 4 * VGROUP_STRIDE)));
+    return __builtin_shufflevector(x0, x1, 0, 1, 2, 3, 4, 5, 6, 7);
   };
+  auto mfma = [](bf16x8 a, bf16x8 b, floatx4 acc) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc, 0, 0, 0); };
+  const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
-  auto zero16 = [] {
-    floatx16 z;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) z[e] = 0.f;
-    return z;
-  };
   // ----- unscheduled pieces, used at the edges of a wavefront's key range
-  // K operands of a 32-key block: `delta` = its tile's ring slot minus the slot kb[] points to
+  // K operands of a 32-key block, ka[2 * ks + kt] in the order the MFMAs take them: `delta` = its
+  // tile's ring slot minus the slot kb[] points to
   auto load_ka = [&](bf16x8 (&ka)[8], int delta, int half) {
 #pragma unroll
-    for (int g = 0; g < 8; ++g) ka[g] = kread_at(kb[g >> 1] + delta, 32 * (g & 1) + half);
+    for (int f = 0; f < 8; ++f) ka[f] = kread_at(kb[f >> 1] + delta, (f & 1) * 4 * GROUP_STRIDE + half);
   };
-  auto mask_block = [&](floatx16& s, int kb32) {
+  auto mask_block = [&](floatx4 (&s)[2][2], int kb32) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      int key = kb32 + 8 * (e >> 2) + 4 * h32 + (e & 3);
-      if (!key_visible(key, kpre, lo_l, hi_l)) s[e] = -INFINITY;
-    }
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = kb32 + 16 * kt + 4 * g4 + e;
+          if (!key_visible(key, kpre, lo_l[qt], hi_l[qt])) s[kt][qt][e] = -INFINITY;
+        }
   };
-  auto block_max = [&](const floatx16& s) {
-    float m0 = fmaxf(fmaxf(s[0], s[1]), s[2]);
-    m0 = fmaxf(fmaxf(m0, s[3]), s[4]);
-    m0 = fmaxf(fmaxf(m0, s[5]), s[6]);
-    float m1 = fmaxf(fmaxf(s[8], s[9]), s[10]);
-    m1 = fmaxf(fmaxf(m1, s[11]), s[12]);
-    m1 = fmaxf(fmaxf(m1, s[13]), s[14]);
-    return lane_xor32_max(fmaxf(fmaxf(m0, s[7]), fmaxf(m1, s[15])));
+  // this lane's part of a block's maximum for query tile qt, and the whole of it
+  auto lane_max = [&](const floatx4 (&s)[2][2], int qt) {
+    const float a = fmaxf(fmaxf(s[0][qt][0], s[0][qt][1]), fmaxf(s[0][qt][2], s[0][qt][3]));
+    const float b = fmaxf(fmaxf(s[1][qt][0], s[1][qt][1]), fmaxf(s[1][qt][2], s[1][qt][3]));
+    return fmaxf(a, b);
+  };
+  auto block_max = [&](const floatx4 (&s)[2][2], float (&mx)[2]) {
+    mx[0] = lane_quad_max(lane_max(s, 0));
+    mx[1] = lane_quad_max(lane_max(s, 1));
   };
   // EXACT mode: what can happen to a freshly computed block of raw scores q.k before it is
-  // exponentiated as exp2(score * c - mref); all of it is rare.  `mx` is the block maximum of the
-  // raw scores.  Lanes l and l + 32 hold the same query (disjoint keys, shared accumulators), so
-  // every decision here is taken per query: mx and the running sum are exchanged between the halves.
-  auto settle = [&](floatx16& nxt, float mx, bool masked, int kb32) {
+  // exponentiated as exp2(score * c - mref); all of it is rare.  `mx` are the block maxima of the
+  // raw scores of the lane's two queries.  Four lanes hold a query (disjoint keys and head dims),
+  // so every decision here is taken per query: maximum and running sum are taken over the four.
+  auto settle = [&](floatx4 (&nxt)[2][2], float (&mx)[2], bool masked, int kb32) {
     if (masked) {  // block cut by a bound: mask in place, then redo the maximum
       mask_block(nxt, kb32);
-      mx = block_max(nxt);
+      block_max(nxt, mx);
     }
-    const float mxs = __builtin_fmaf(mx, c, -mref);  // block maximum in exponent units
-    if (__builtin_amdgcn_ballot_w64(__builtin_fabsf(mxs) > 60.f) == 0) return;  // the usual case
-    const float l_run = lane_xor32_sum(l_acc[0] + l_acc[1]);  // of the query, not of this lane's keys
-    const bool need = mxs > 60.f || (l_run == 0.f && mxs < -60.f && mxs > -INFINITY);
-    if (__builtin_amdgcn_ballot_w64(need) != 0) {
-      const float delta = need ? mxs : 0.f;
-      const float alpha = l_run == 0.f ? 1.f : __builtin_amdgcn_exp2f(-delta);
-      mref += delta;
-      l_acc[0] *= alpha;
-      l_acc[1] *= alpha;
+    const float mxs[2] = {__builtin_fmaf(mx[0], c, -mref[0]), __builtin_fmaf(mx[1], c, -mref[1])};  // in exponent units
+    if (__builtin_amdgcn_ballot_w64(fmaxf(__builtin_fabsf(mxs[0]), __builtin_fabsf(mxs[1])) > 60.f) == 0) return;  // the usual case
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+    for (int qt = 0; qt < 2; ++qt) {
+      const float l_run = lane_quad_sum(l_acc[qt]);  // of the query, not of this lane's keys
+      const bool need = mxs[qt] > 60.f || (l_run == 0.f && mxs[qt] < -60.f && mxs[qt] > -INFINITY);
+      if (__builtin_amdgcn_ballot_w64(need) != 0) {
+        const float delta = need ? mxs[qt] : 0.f;
+        const float alpha = l_run == 0.f ? 1.f : __builtin_amdgcn_exp2f(-delta);
+        mref[qt] += delta;
+        l_acc[qt] *= alpha;
 #pragma unroll
-        for (int e = 0; e < 16; ++e) oacc[db][e] *= alpha;
+        for (int dt = 0; dt < 8; ++dt) oacc[dt][qt] *= alpha;
+      }
     }
   };
   // a freshly computed block of scores, before its weights are formed
-  auto finish_scores = [&](floatx16& nxt, float mx, bool masked, int kb32) {
+  auto finish_scores = [&](floatx4 (&nxt)[2][2], float (&mx)[2], bool masked, int kb32) {
     if (FAST) {
       if (masked) mask_block(nxt, kb32);
     } else {
@@ -547,73 +582,79 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     }
   };
 
-  // ----- hand-scheduled step: QK^T of the next key block (8 MFMAs) and PV of the current one
-  // (8 MFMAs) with the softmax VALU work spread between them.  One "slot" is one MFMA.  LDS
-  // operands are fetched a whole phase (8 slots) ahead: the V^T operands of this step's PV during
-  // its QK^T slots, the K operands of the NEXT step's QK^T during this step's PV slots (ka lives
-  // across steps and across the tile barrier: the K tile it reads was made visible by an earlier
-  // barrier and is not overwritten before the next one).  The exponentials of the current block
-  // run one bf16 pair per slot in slots 0..7, the packing + row sums one slot later; in EXACT mode
-  // the maximum of the next block is taken in the PV slots once its MFMA chain has drained.
-  // sched_barrier keeps the compiler from regrouping the slots.
+  // ----- hand-scheduled step: QK^T of the next key block (16 MFMAs) and PV of the current one
+  // (16 MFMAs) with the softmax VALU work spread between them.  One "slot" is one MFMA.  LDS
+  // operands are fetched about a phase ahead: the V^T operands of this step's PV during its QK^T
+  // slots, the K operands of the NEXT step's QK^T during the second half of this step's PV slots
+  // (ka lives across steps and across the tile barrier: the K tile it reads was made visible by an
+  // earlier barrier and is not overwritten before the next one).  The score accumulators are the
+  // B operand of PV as they stand: the lane's 8 weights of query tile qt, packed to bf16, are
+  // keys 4*g4 .. +3 and 16 + 4*g4 .. +3 of the block, the numbering the V^T reads follow.  PV
+  // runs query tile 0 first, so the weights of query tile 1 are only needed 8 slots later: the
+  // exponentials of the 8 bf16 pairs are spread over slots 0..20 of the 32, the packing + row sums
+  // follow two slots behind, and in EXACT mode the maximum of the next block is taken in the last
+  // PV slots once its MFMA chain has drained.  sched_barrier keeps the compiler from regrouping
+  // the slots.
   bf16x8 ka[8];
-  // HALF: byte offset of the block's half inside its tile for the V reads (block j) and the K reads
-  // (block j + 2, one tile further): 0 or BLOCK32, the same for both.
-  auto steady = [&](const floatx16& s, floatx16& n, auto half_c, bool mask_next, int kb32_next) {
+  // HALF: which half of its tile the V reads (block j) and the K reads (block j + 2, one tile
+  // further) address: the same for both.
+  auto steady = [&](const floatx4 (&s)[2][2], floatx4 (&n)[2][2], auto half_c, bool mask_next, int kb32_next) {
     constexpr int HALF = decltype(half_c)::value;
     bf16x8 va[8], pb[2];
     float px[8][2];
+    // pair u = 4 * qt + 2 * kt + h: weights of keys 16 * kt + 4 * g4 + 2 * h, + 1 for query tile qt
     auto stage_e = [&](int u) {
+      const int qt = u >> 2, kt = (u >> 1) & 1, h = u & 1;
       if (FAST) {
-        px[u][0] = __builtin_amdgcn_exp2f(s[2 * u]);
-        px[u][1] = __builtin_amdgcn_exp2f(s[2 * u + 1]);
+        px[u][0] = __builtin_amdgcn_exp2f(s[kt][qt][2 * h]);
+        px[u][1] = __builtin_amdgcn_exp2f(s[kt][qt][2 * h + 1]);
       } else {
-        px[u][0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u], c, -mref));
-        px[u][1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * u + 1], c, -mref));
+        px[u][0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][qt][2 * h], c, -mref[qt]));
+        px[u][1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][qt][2 * h + 1], c, -mref[qt]));
       }
     };
     auto stage_c = [&](int u) {
       floatx2 f = {px[u][0], px[u][1]};
-      bf16x2 h = __builtin_convertvector(f, bf16x2);
-      l_acc[u & 1] = __builtin_amdgcn_fdot2_f32_bf16(h, ones2, l_acc[u & 1], false);  // sums what PV multiplies
-      pb[u >> 2][2 * (u & 3)] = h[0];
-      pb[u >> 2][2 * (u & 3) + 1] = h[1];
+      bf16x2 h2 = __builtin_convertvector(f, bf16x2);
+      l_acc[u >> 2] = __builtin_amdgcn_fdot2_f32_bf16(h2, ones2, l_acc[u >> 2], false);  // sums what PV multiplies
+      pb[u >> 2][2 * (u & 3)] = h2[0];
+      pb[u >> 2][2 * (u & 3) + 1] = h2[1];
     };
-    // exp2 of pair u is issued in slot e_slot(u), packed one slot later: pairs 0-3 (P^T half 0,
-    // needed from slot 8) in every other QK^T slot, pairs 4-7 (half 1, needed from slot 12) in
-    // slots 7..10, the maximum of the new block in slots 12..15.  Both phases then carry about
-    // the same VALU load per MFMA, which matters because the two wavefronts of a SIMD tend to
-    // be in the same phase.
+    // slot (0..31, PV slots from 16) in which the exponentials of pair u are issued
     auto valu_slot = [&](int k) {
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
-        const int es = u < 4 ? 2 * u : u + 3;
+        const int es = u < 4 ? 4 * u : 2 * u + 6;
         if (es == k) stage_e(u);
-        if (es + 1 == k) stage_c(u);
+        if (es + 2 == k) stage_c(u);
       }
     };
 #pragma unroll
-    for (int g = 0; g < 8; ++g) {
-      va[g] = vread_at(vb[g & 3], (g >> 2) * 4 * GROUP_STRIDE + HALF);
-      n = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[g], qf[g], g == 0 ? zero16() : n, 0, 0, 0);
-      valu_slot(g);
+    for (int k = 0; k < 16; ++k) {  // QK^T: k-step ks, key tile kt, query tile qt
+      const int ks = k >> 2, kt = (k >> 1) & 1, qt = k & 1;
+      if ((k & 1) == 0) va[k >> 1] = vread_at(vb[k >> 2], 32 * ((k >> 1) & 1) + HALF * VBLOCK32);
+      n[kt][qt] = mfma(ka[2 * ks + kt], qf[qt][ks], ks == 0 ? zero4 : n[kt][qt]);
+      valu_slot(k);
       __builtin_amdgcn_sched_barrier(0);
     }
-    float m0 = 0.f, m1 = 0.f;
+    float m[2] = {0.f, 0.f};
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      ka[j] = kread_at(kb[j >> 1], 32 * (j & 1) + HALF);
-      oacc[j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[j], pb[j >> 2], oacc[j & 3], 0, 0, 0);
-      valu_slot(8 + j);
+    for (int k = 0; k < 16; ++k) {  // PV: query tile qt, head-dim tile dt
+      const int qt = k >> 3, dt = k & 7;
+      if (k >= 8) ka[k - 8] = kread_at(kb[(k - 8) >> 1], (k & 1) * 4 * GROUP_STRIDE + HALF * BLOCK32);
+      oacc[dt][qt] = mfma(va[dt], pb[qt], oacc[dt][qt]);
+      valu_slot(16 + k);
       if (!FAST) {
-        if (j == 4) m0 = fmaxf(fmaxf(n[0], n[1]), fmaxf(n[2], n[3]));
-        if (j == 5) m0 = fmaxf(fmaxf(m0, n[4]), fmaxf(n[5], fmaxf(n[6], n[7])));
-        if (j == 6) m1 = fmaxf(fmaxf(n[8], n[9]), fmaxf(n[10], n[11]));
-        if (j == 7) m1 = fmaxf(fmaxf(m1, n[12]), fmaxf(n[13], fmaxf(n[14], n[15])));
+        if (k == 12) m[0] = lane_max(n, 0);
+        if (k == 14) m[1] = lane_max(n, 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    finish_scores(n, FAST ? 0.f : lane_xor32_max(fmaxf(m0, m1)), mask_next, kb32_next);
+    if (!FAST) {
+      m[0] = lane_quad_max(m[0]);
+      m[1] = lane_quad_max(m[1]);
+    }
+    finish_scores(n, m, mask_next, kb32_next);
   };
 
   // Step j: softmax + PV of key block j (scores in `cur`, V rows in the current tile) and QK^T of
@@ -636,16 +677,16 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     }
   }
   auto needs_mask = [&](int j) { return !block_unmasked(wb, kpre, kt_lo + 32 * j); };
-  // half_c: which half of its tile block j is (0 / BLOCK32).  Block j + 1 is the other half of the
-  // same tile (half 0) or the first half of the next tile (half BLOCK32).
-  auto step = [&](int j, floatx16& cur, floatx16& nxt, auto half_c, auto with_loader, int free_slot) {
+  // half_c: which half of its tile block j is (0 / 1).  Block j + 1 is the other half of the same
+  // tile (half 0) or the first half of the next tile (half 1).
+  auto step = [&](int j, floatx4 (&cur)[2][2], floatx4 (&nxt)[2][2], auto half_c, auto with_loader, int free_k, int free_v) {
     constexpr int HALF = decltype(half_c)::value;
-    if (decltype(with_loader)::value) feed_tile(free_slot);
+    if (decltype(with_loader)::value) feed_tile(free_k, free_v);
     const bool in1 = j >= jq1 && j <= jp1, in2 = j >= jq2 && j <= jp2;
     if (!in1 && !in2) return;
     if (j == jq1 || (in2 && j == jq2)) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) cur[e] = -INFINITY;
+      for (int t = 0; t < 4; ++t) cur[t >> 1][t & 1] = floatx4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
       if (HALF == 0) load_ka(ka, k0 - k1, BLOCK32);  // second half of the current tile
       else load_ka(ka, 0, 0);                         // first half of the next tile
     }
@@ -662,21 +703,27 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   // tile work: the first reads Q out of LDS, the second computes the scores of key block 0.
   // ---------------------------------------------------------------- slot -1: the first key tile has landed
   slot_barrier(in_flight);
-  feed_tile(k3);
+  feed_tile(k3, v3);
   if (jq1 < 0 && jp1 >= 0) {  // scores of key block 0, ahead of the pipeline (the tile sits in slot k1)
     load_ka(ka, 0, 0);
-    s0 = zero16();
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[ks], qf[ks], s0, 0, 0, 0);
-    finish_scores(s0, FAST ? 0.f : block_max(s0), needs_mask(0), kt_lo);
+    for (int t = 0; t < 4; ++t) s0[t >> 1][t & 1] = zero4;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int ks = k >> 2, kt = (k >> 1) & 1, qt = k & 1;
+      s0[kt][qt] = mfma(ka[2 * ks + kt], qf[qt][ks], s0[kt][qt]);
+    }
+    float mx[2] = {0.f, 0.f};
+    if (!FAST) block_max(s0, mx);
+    finish_scores(s0, mx, needs_mask(0), kt_lo);
     load_ka(ka, 0, BLOCK32);
   }
   rotate();
   INTRA_DIAG(const long long t_d = wall_clock64(); const long long c_d = __builtin_readcyclecounter();)
   slot_barrier(in_flight);  // opens tile 0; the held stores went out after the request for tile 1
   for (int i = 0;;) {
-    step(2 * i, s0, s1, ic<0>{}, ic<1>{}, k3);
-    step(2 * i + 1, s1, s0, ic<BLOCK32>{}, ic<0>{}, 0);
+    step(2 * i, s0, s1, ic<0>{}, ic<1>{}, k3, v3);
+    step(2 * i + 1, s1, s0, ic<1>{}, ic<0>{}, 0, 0);
     rotate();
     if (++i == ntiles) break;
     tile_barrier<PER_TILE>();
@@ -693,47 +740,50 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   // (idle wavefronts run through it as well and hold nothing: the registers of the held output
   // are then rewritten in every work item and free during the tile loop)
   {
-  const float l_tot = lane_xor32_sum(l_acc[0] + l_acc[1]);
+  const float l_tot[2] = {lane_quad_sum(l_acc[0]), lane_quad_sum(l_acc[1])};
   if (FAST) {
     // Weights were formed without a reference: the result is good iff the weight sum stayed inside
     // 2^-100 .. 2^60 (no weight overflowed, and the largest ones are far from underflow).  The
     // integer comparison of the bit patterns also catches a negative or NaN sum.
-    const uint32_t lb = __float_as_uint(l_tot);
-    const bool bad = wave_active && row_valid && !(lb >= 0x0d800000u && lb <= 0x5d800000u);
+    const uint32_t lb0 = __float_as_uint(l_tot[0]), lb1 = __float_as_uint(l_tot[1]);
+    const bool bad = wave_active && ((row_valid[0] && !(lb0 >= 0x0d800000u && lb0 <= 0x5d800000u)) ||
+                                     (row_valid[1] && !(lb1 >= 0x0d800000u && lb1 <= 0x5d800000u)));
     if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0)
       __hip_atomic_fetch_or(&redo[(cw.round >> 5) & (REDO_WORDS - 1)], 1u << (cw.round & 31), __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_WORKGROUP);
   }
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2; lanes of clamped rows repeat their row's value
+  const float inv[2] = {l_tot[0] > 0.f ? 1.f / l_tot[0] : 0.f, l_tot[1] > 0.f ? 1.f / l_tot[1] : 0.f};
+  // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2; the lane quarters g4 = 0, 1 store the values of
+  // query tiles 0, 1, the other two (and lanes of clamped rows) repeat them
   held = wave_active ? (p.lse != nullptr ? 9 : 8) : 0;
-  lse_dst = p.lse + (batch * p.lse_bs + hq * p.lse_hs + qpos * p.lse_ts);
-  lse_val = (mref + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
-  // Lane l and lane l+32 hold the same query: per 16 head dims the lower lane has dims 0-3 and
-  // 8-11, the upper one 4-7 and 12-15.  One permlane32 swap per register pair turns that into
-  // dims 0-7 / 8-15, i.e. 16-byte chunk 2*ks + h of the row for ks = 2*db + g2; pair_exchange
-  // then regroups the chunks so that four lanes store 64 contiguous bytes of one row.
+  {
+    const int qt = g4 & 1;
+    lse_dst = p.lse + (batch * p.lse_bs + hq * p.lse_hs + (qt ? qpos[1] : qpos[0]) * p.lse_ts);
+    lse_val = ((qt ? mref[1] : mref[0]) + __builtin_amdgcn_logf(qt ? l_tot[1] : l_tot[0])) * 0.6931471805599453f;
+  }
+  // The four lanes of a query hold head dims 4 * g4 .. + 3 of every 16-dim tile.  For the tile pair
+  // 2m, 2m+1 a lane quarter and its neighbour (g4 ^ 1) trade 8 bytes: the even one keeps its 4 dims
+  // of tile 2m and receives the neighbour's (the next 4 dims), the odd one does the same for tile
+  // 2m+1.  Each lane then owns one whole 16-byte chunk of the row: 4m + 2 * (g4 % 2) + g4 / 2.
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
-    for (int g2 = 0; g2 < 2; ++g2) {
-      uint32_t w[4];
+    for (int m = 0; m < 4; ++m) {
+      uint32_t w[2][2];
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int k = 0; k < 2; ++k) {
-          const int e = 8 * g2 + 4 * half + 2 * k;
-          floatx2 f = {oacc[db][e] * inv, oacc[db][e + 1] * inv};
-          w[2 * half + k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+          floatx2 f = {oacc[2 * m + t][qt][2 * k] * inv[qt], oacc[2 * m + t][qt][2 * k + 1] * inv[qt]};
+          w[t][k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
         }
-      auto r0 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
-      auto r1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
-      pk[2 * db + g2] = u32x4{r0[0], r1[0], r0[1], r1[1]};
+      auto r0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
+      auto r1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
+      pk[4 * qt + m] = u32x4{r0[0], r1[0], r0[1], r1[1]};
     }
-  pair_exchange(pk);
-  const int64_t ohead = batch * p.o_bs + hq * p.o_hs + (2 * qpar + h32) * 8;
-  orow_a = p.o + (ohead + opos_a * p.o_rs);
-  orow_b = p.o + (ohead + opos_b * p.o_rs);
+  const int64_t ohead = batch * p.o_bs + hq * p.o_hs + (2 * (g4 & 1) + (g4 >> 1)) * 8;
+  orow[0] = p.o + (ohead + qpos[0] * p.o_rs);
+  orow[1] = p.o + (ohead + qpos[1] * p.o_rs);
   }
   INTRA_DIAG(dg[0] += t_b - t_a; dg[1] += t_c - t_b; dg[2] += t_d - t_c; dg[3] += t_e - t_d;
              dg[4] += wall_clock64() - t_e; dg[5] += 1; dg[6] += ntiles;)

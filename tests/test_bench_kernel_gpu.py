@@ -71,9 +71,10 @@ def test_image_rows(tmp_path):
 
 def test_ceiling_and_phases_modes(tmp_path):
     doc, _ = run_cli(tmp_path, "ceiling")
-    const, rand = doc["rows"]
-    assert const["operands"].startswith("constant") and 0 < rand["tflops"] <= const["tflops"] * 1.02 <= PEAK * 1.05
-    assert 1000 < rand["shader_clock_mhz"] <= const["shader_clock_mhz"] * 1.02 < 2600
+    assert [r["mfma"] for r in doc["rows"]] == ["16x16x32", "16x16x32", "32x32x16", "32x32x16"]
+    for const, rand in (doc["rows"][:2], doc["rows"][2:]):
+        assert const["operands"].startswith("constant") and 0 < rand["tflops"] <= const["tflops"] * 1.02 <= PEAK * 1.05
+        assert 1000 < rand["shader_clock_mhz"] <= const["shader_clock_mhz"] * 1.02 < 2600
     from intra_amd import _lib
     doc, _ = run_cli(tmp_path, "phases", "--pattern", "scatter", "--seqlen", "8192", "--iters", "3", "--warmup", "1",
                      lib=_lib.DIAG_LIB_PATH)
