@@ -246,9 +246,9 @@ int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint
  * INTRA_ERR_UNSUPPORTED and never touches such a buffer.
  *
  * intra_diag_mfma_ceiling: one launch of `workgroups` x 8 wavefronts that issue nothing but bf16
- * MFMAs on independent accumulators: `shape` 16 = v_mfma_f32_16x16x32_bf16 (the forward kernel's
- * instruction, 32 per iteration and wavefront), 32 = v_mfma_f32_32x32x16_bf16 (the backward
- * kernels', 16 per iteration), on
+ * MFMAs on independent accumulators: `shape` 16 = v_mfma_f32_16x16x32_bf16 (the kernels'
+ * instruction, 32 per iteration and wavefront), 32 = v_mfma_f32_32x32x16_bf16 (the alternative
+ * shape, 16 per iteration), on
  * operands read once from `table` (131072 bytes the caller fills: constant or random bf16 bits).
  * `sink` takes workgroups * 512 floats, `clocks` per workgroup {shader cycles, 100 MHz ticks} of
  * the loop.  Work per launch: workgroups * 8 * iters * 16 * 32768 flop.  Allocates nothing. */

@@ -288,7 +288,7 @@ def bench_phases(args):
 
 def bench_ceiling(args):
     """MFMA-only launches (8 wavefronts per CU on every CU, nothing but v_mfma_f32_16x16x32_bf16, the
-    forward kernel's instruction, or v_mfma_f32_32x32x16_bf16, the backward kernels') with constant
+    kernels' instruction, or v_mfma_f32_32x32x16_bf16, the alternative shape) with constant
     and with random operand bits: TFLOP/s and the shader clock each ran at."""
     lib = _lib.load()
     n_wg = torch.cuda.get_device_properties(0).multi_processor_count

@@ -22,8 +22,6 @@
 
 namespace intra {
 
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
 enum BwdMode : int { BWD_DQ = 0, BWD_DK = 1, BWD_DV = 2 };
 
 struct BParams {
@@ -46,11 +44,17 @@ struct BParams {
   int bundle;        // pairs of one XCD that are worked on together
 };
 
-constexpr int BWD_SLOT = 2 * TILE_BYTES + 512;  // two tiles and 2 x 64 column scalars
+constexpr int BWD_SLOT = 2 * FTILE + 512;  // two tiles and 2 x 64 column scalars
 constexpr int BWD_LDS_BYTES = 3 * BWD_SLOT;
 
 // RMAP: row map (intra_bwd_maps.h).  PARTIAL: the results are partial sums over the set's columns,
 // written as fp32 to p.part instead of bf16 to dk / dv (sink pass).
+//
+// MFMA layout (v_mfma_f32_16x16x32_bf16, as in the forward kernel): a block of 32 columns times the
+// wavefront's 32 rows is 2 x 2 tiles [ct][rt] with 4 k-steps; lane (l16 = lane % 16, g4 = lane / 16)
+// holds columns 16*ct + 4*g4 .. +3 of row 16*rt + l16.  The packed weights of a row tile are the B
+// operand of the accumulation, whose 32-column reduction is numbered slot s of lane quarter g4 =
+// column 16*(s/4) + 4*g4 + s%4; the transposing reads of the X tile follow that numbering.
 template <class RMAP, int MODE, int HP, bool PARTIAL = false>
 __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   constexpr int NW = 8;
@@ -63,8 +67,8 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int h32 = lane >> 5;
-  const int l32 = lane & 31;
+  const int l16 = lane & 15;
+  const int g4 = lane >> 4;
 
   // ---------------------------------------------------------------- work item
   // Workgroups start in blockIdx order, round-robin over the 8 XCDs, and a CU takes the next one
@@ -102,18 +106,27 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   const int ntiles = ce >= cb ? (ce - cb + BN) / BN : 0;
 
   // ---------------------------------------------------------------- this wavefront's rows
+  // a lane works for two rows: 16 * rt + l16 of the wavefront's 32 (rows past the end repeat the last)
   const int hw = ROWS_ARE_QUERIES ? wave % HP : 0;
   const int wr0 = r0 + (ROWS_ARE_QUERIES ? wave / HP : wave) * 32;
   const bool wave_active = wr0 <= r1;
-  const bool row_valid = wr0 + l32 <= r1;
-  const int row = im_min(wr0 + l32, r1);
-  const int lo_l = map.lo(row), hi_l = map.hi(row);
-  // union and intersection of the ranges of the wavefront's rows (rows past the end repeat the last)
+  bool row_valid[2];
+  int row[2], lo_l[2], hi_l[2];
+  int64_t rpos[2];
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
+    row_valid[rt] = wr0 + 16 * rt + l16 <= r1;
+    row[rt] = im_min(wr0 + 16 * rt + l16, r1);
+    lo_l[rt] = map.lo(row[rt]);
+    hi_l[rt] = map.hi(row[rt]);
+    rpos[rt] = map.row_pos(row[rt]);
+  }
+  // union and intersection of the ranges of the wavefront's rows
   WaveBounds wb;
   {
-    int a = lo_l, b = hi_l, c = lo_l, d = hi_l;
+    int a = im_min(lo_l[0], lo_l[1]), b = im_max(hi_l[0], hi_l[1]), c = im_max(lo_l[0], lo_l[1]), d = im_min(hi_l[0], hi_l[1]);
 #pragma unroll
-    for (int m = 1; m < 32; m <<= 1) {
+    for (int m = 1; m < 16; m <<= 1) {
       a = im_min(a, __shfl_xor(a, m));
       b = im_max(b, __shfl_xor(b, m));
       c = im_max(c, __shfl_xor(c, m));
@@ -129,71 +142,79 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   const bool any = wave_active && wb.w_hi >= cb && (kpre > 0 || wb.w_hi >= wb.w_lo);  // (early rows may meet prefix columns only)
   const int jb_lo = !any ? 1 : kpre > 0 ? 0 : (im_max(wb.w_lo, cb) - cb) >> 5;
   const int jb_hi = !any ? 0 : (wb.w_hi - cb) >> 5;
-  const int64_t rpos = map.row_pos(row);
   const int hq = kvh * p.ratio + hg * HP + hw;  // query head of a query row
 
   // ---------------------------------------------------------------- row operands (MFMA B fragments)
-  // lane holds row l32, head dims 16*ks + 8*h32 .. +7 for ks = 0..7
-  bf16x8 r1f[8], r2f[8];
-  float L2_row = 0.f, D_row = 0.f;
-  {
+  // [rt][ks]: lane holds row 16 * rt + l16, head dims 32 * ks + 8 * g4 .. +7
+  bf16x8 r1f[2][4], r2f[2][4];
+  float L2_row[2] = {0.f, 0.f}, D_row[2] = {0.f, 0.f};
+#pragma unroll
+  for (int rt = 0; rt < 2; ++rt) {
     const uint16_t *a1, *a2;
     if (ROWS_ARE_QUERIES) {
-      a1 = p.q + (batch * p.q_bs + rpos * p.q_rs + hq * p.q_hs + h32 * 8);
-      a2 = p.dout + (batch * p.do_bs + rpos * p.do_rs + hq * p.do_hs + h32 * 8);
+      a1 = p.q + (batch * p.q_bs + rpos[rt] * p.q_rs + hq * p.q_hs + g4 * 8);
+      a2 = p.dout + (batch * p.do_bs + rpos[rt] * p.do_rs + hq * p.do_hs + g4 * 8);
     } else {
-      a1 = p.k + (batch * p.k_bs + rpos * p.k_rs + kvh * p.k_hs + h32 * 8);
-      a2 = p.v + (batch * p.v_bs + rpos * p.v_rs + kvh * p.v_hs + h32 * 8);
+      a1 = p.k + (batch * p.k_bs + rpos[rt] * p.k_rs + kvh * p.k_hs + g4 * 8);
+      a2 = p.v + (batch * p.v_bs + rpos[rt] * p.v_rs + kvh * p.v_hs + g4 * 8);
     }
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      r1f[ks] = *reinterpret_cast<const bf16x8*>(a1 + ks * 16);
-      if (MODE != BWD_DV) r2f[ks] = *reinterpret_cast<const bf16x8*>(a2 + ks * 16);
+    for (int ks = 0; ks < 4; ++ks) {
+      r1f[rt][ks] = *reinterpret_cast<const bf16x8*>(a1 + ks * 32);
+      if (MODE != BWD_DV) r2f[rt][ks] = *reinterpret_cast<const bf16x8*>(a2 + ks * 32);
     }
     if (ROWS_ARE_QUERIES) {
-      // D = dO . O of the row: this lane's 64 head dims, then the other half from lane ^ 32
-      const uint16_t* ao = p.o + (batch * p.o_bs + rpos * p.o_rs + hq * p.o_hs + h32 * 8);
+      // D = dO . O of the row: this lane's 32 head dims, then the rest from the other three lanes of the row
+      const uint16_t* ao = p.o + (batch * p.o_bs + rpos[rt] * p.o_rs + hq * p.o_hs + g4 * 8);
       float part = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 of = *reinterpret_cast<const bf16x8*>(ao + ks * 16);
+      for (int ks = 0; ks < 4; ++ks) {
+        const bf16x8 of = *reinterpret_cast<const bf16x8*>(ao + ks * 32);
 #pragma unroll
-        for (int d = 0; d < 8; ++d) part += (float)r2f[ks][d] * (float)of[d];
+        for (int d = 0; d < 8; ++d) part += (float)r2f[rt][ks][d] * (float)of[d];
       }
-      D_row = lane_xor32_sum(part);
-      L2_row = p.lse[batch * p.lse_bs + hq * p.lse_hs + rpos * p.lse_ts] * 1.4426950408889634f;
-      if (row_valid && h32 == 0) p.dsum[batch * p.ds_bs + hq * p.ds_hs + rpos] = D_row;
+      D_row[rt] = lane_quad_sum(part);
+      L2_row[rt] = p.lse[batch * p.lse_bs + hq * p.lse_hs + rpos[rt] * p.lse_ts] * 1.4426950408889634f;
+      if (row_valid[rt] && g4 == 0) p.dsum[batch * p.ds_bs + hq * p.ds_hs + rpos[rt]] = D_row[rt];
     }
   }
 
   // ---------------------------------------------------------------- LDS addressing (as in the forward kernel)
   const int ld_row = lane >> 4;
   const uint32_t ld_col = (((lane & 15) ^ (4 * ld_row)) << 4);
-  int kaddr[8];
+  int kaddr[4];
+  {
+    const int r = l16 & 3;
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks)
-    kaddr[ks] = (l32 >> 2) * GROUP_STRIDE + (l32 & 3) * 256 + (((2 * ks + h32) ^ (4 * (l32 & 3))) << 4);
+    for (int ks = 0; ks < 4; ++ks) kaddr[ks] = (l16 >> 2) * FGROUP_STRIDE + r * 256 + 64 * (ks ^ r) + 16 * g4;
+  }
   int vaddr[4];
   {
-    const int i16 = lane & 15, g2 = (lane >> 4) & 1, ri = i16 >> 2;
+    const int ri = l16 >> 2;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
-      vaddr[db] = h32 * GROUP_STRIDE + ri * 256 + (((4 * db + 2 * g2 + ((i16 & 3) >> 1)) ^ (4 * ri)) << 4) + 8 * (i16 & 1);
+    for (int a = 0; a < 4; ++a)
+      vaddr[a] = g4 * FGROUP_STRIDE + ri * 256 + 64 * (a ^ ri) + 16 * ((l16 & 3) >> 1) + 8 * (l16 & 1);
   }
-  auto kread = [&](int off, int ks) { return *reinterpret_cast<const bf16x8*>(smem + off + kaddr[ks]); };
-  auto vread = [&](int off, int j) {
-    const int o2 = off + vaddr[j & 3] + (j >> 2) * 4 * GROUP_STRIDE;
+  // row-per-lane operand 2 * ks + ct of a 32-row block: rows 16 * ct + l16, head dims of k-step ks
+  auto kread = [&](int off, int f) {
+    return *reinterpret_cast<const bf16x8*>(smem + off + kaddr[f >> 1] + (f & 1) * 4 * FGROUP_STRIDE);
+  };
+  // transposed operand: head dims 16 * dt .. + 15 of the block's 32 rows
+  auto vread = [&](int off, int dt) {
+    const int o2 = off + vaddr[dt >> 1] + 32 * (dt & 1);
     bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(smem + o2));
     bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (__attribute__((address_space(3))) bf16x4*)(smem + o2 + 2 * GROUP_STRIDE));
+        (__attribute__((address_space(3))) bf16x4*)(smem + o2 + 4 * FGROUP_STRIDE));
     return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
   };
+  auto mfma = [](bf16x8 a, bf16x8 b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); };
+  const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
-  floatx16 acc[4];
+  floatx4 acc[8][2];  // [head-dim tile][row tile]: head dims 16 * dt + 4 * g4 .. + 3 of row 16 * rt + l16
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[db][e] = 0.f;
+    for (int rt = 0; rt < 2; ++rt) acc[dt][rt] = zero4;
   const float c2 = p.scale_log2;
   const float s_hidden = c2 >= 0.f ? -INFINITY : INFINITY;  // score that gives exp2(s * c2 - lse) = 0
 
@@ -239,9 +260,9 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
       const int grp = wave * 2 + gi;
       const int c = im_min(cb + cu.tile * BN + 4 * grp + ld_row, n_cols - 1);
       const uint32_t pos = col_pos(c);
-      dma_group(c1base + (cu.head * c1hs + (uint64_t)pos * c1rs + ld_col), lds_base + slot_off + grp * GROUP_STRIDE);
+      dma_group(c1base + (cu.head * c1hs + (uint64_t)pos * c1rs + ld_col), lds_base + slot_off + grp * FGROUP_STRIDE);
       dma_group(c2base + (cu.head * c2hs + (uint64_t)pos * c2rs + ld_col),
-                lds_base + slot_off + TILE_BYTES + grp * GROUP_STRIDE);
+                lds_base + slot_off + FTILE + grp * FGROUP_STRIDE);
     }
   };
   // column scalars of a step (dK / dV): wavefront 0 fetches lse * log2(e) and D of its 64 columns
@@ -257,22 +278,21 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   };
   auto put_scalars = [&](int slot_off) {
     if (!ROWS_ARE_QUERIES && wave == 0) {
-      float* sc = reinterpret_cast<float*>(smem + slot_off + 2 * TILE_BYTES);
+      float* sc = reinterpret_cast<float*>(smem + slot_off + 2 * FTILE);
       sc[lane] = sc_l;
       sc[64 + lane] = sc_d;
     }
   };
-  auto zero16 = [] {
-    floatx16 z;
+  // scores of a block whose rows start at LDS offset `off`, outside the schedule
+  auto scores = [&](int off, floatx4 (&s)[2][2]) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) z[e] = 0.f;
-    return z;
-  };
-  auto scores = [&](int off) {
-    floatx16 s = zero16();
+    for (int t = 0; t < 4; ++t) s[t >> 1][t & 1] = zero4;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kread(off, ks), r1f[ks], s, 0, 0, 0);
-    return s;
+    for (int f = 0; f < 8; ++f) {
+      const bf16x8 a = kread(off, f);
+#pragma unroll
+      for (int rt = 0; rt < 2; ++rt) s[f & 1][rt] = mfma(a, r1f[rt][f >> 1], s[f & 1][rt]);
+    }
   };
 
   // Three tile slots: while step t works on its tile, the tile of step t+1 has landed (the scores
@@ -286,14 +306,16 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
     advance(ld);
   }
   int slot0 = 0, slot1 = BWD_SLOT, slot2 = 2 * BWD_SLOT;
-  floatx16 s_cur;
+  floatx4 s_cur[2][2];  // [ct][rt]
 #pragma unroll
-  for (int e = 0; e < 16; ++e) s_cur[e] = 0.f;
+  for (int t = 0; t < 4; ++t) s_cur[t >> 1][t & 1] = zero4;
   bool have = false;  // s_cur and fr hold what a previous block prepared for the one that comes next
-  constexpr int NSLOT = MODE == BWD_DV ? 16 : 24;  // MFMAs per block
-  constexpr int LA = MODE == BWD_DK ? 4 : MODE == BWD_DV ? 8 : 6;  // slots between the request of an LDS operand and its use
-  static_assert(NSLOT % LA == 0, "a block must leave the ring where the next block expects it");
-  constexpr int W0 = MODE == BWD_DV ? 2 : 10;      // slot of the first weight stage
+  // One slot is one MFMA; an LDS operand serves two consecutive slots (the two row tiles).
+  constexpr int NFRAG = MODE == BWD_DV ? 16 : 24;  // LDS operands per block
+  constexpr int LA = MODE == BWD_DK ? 4 : MODE == BWD_DV ? 8 : 6;  // operands between the request of one and its use
+  static_assert(NFRAG % LA == 0, "a block must leave the ring where the next block expects it");
+  constexpr int WS = MODE == BWD_DV ? 4 : 16;      // slot of the first weight stage
+  constexpr int WSTEP = MODE == BWD_DV ? 1 : 2;    // slots from one stage to the next
   bf16x8 fr[LA];
 #pragma unroll
   for (int i = 0; i < LA; ++i) fr[i] = bf16x8{};
@@ -313,91 +335,103 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
       }
       const int sb_lo = cb + 32 * jb;  // first column of the block
       // maps with a block predicate: a row meets the whole block or nothing of it
-      bool lane_sees = true;
-      uint64_t seeing = ~0ull;
+      bool lane_sees[2] = {true, true};
+      bool masked;
       if (RMAP::kBlockPredicate) {
-        lane_sees = map.sees(row, sb_lo);
-        seeing = __builtin_amdgcn_ballot_w64(lane_sees);
-        if (seeing == 0) {
+        lane_sees[0] = map.sees(row[0], sb_lo);
+        lane_sees[1] = map.sees(row[1], sb_lo);
+        if (__builtin_amdgcn_ballot_w64(lane_sees[0] || lane_sees[1]) == 0) {
           have = false;
           continue;
         }
+        masked = __builtin_amdgcn_ballot_w64(lane_sees[0] && lane_sees[1]) != ~0ull;
+      } else {
+        masked = !block_unmasked(wb, kpre, sb_lo);
       }
-      const bool masked = RMAP::kBlockPredicate ? seeing != ~0ull : !block_unmasked(wb, kpre, sb_lo);
       // this block, the one that follows in this order, and the one after that
-      const int c1off = slot0 + blk * BLOCK32, c2off = c1off + TILE_BYTES;
-      const int c1n = blk == 0 ? c1off + BLOCK32 : slot1, c2n = c1n + TILE_BYTES;
-      const int c1nn = blk == 0 ? slot1 : slot1 + BLOCK32;
-      // Hand-scheduled: one slot is one MFMA.  dQ / dK: slots 0-7 dP of this block, 8-15 the
-      // scores of the next block, 16-23 the accumulation; dV: 0-7 scores of the next block, 8-15
-      // the accumulation.  The LDS operand of slot i is requested in slot i - LA into a ring of
-      // LA fragments, across block and step boundaries (both following blocks have landed); the
-      // weights of element pair u are formed in slot W0 + u, after dP has drained and before the
+      const int c1off = slot0 + blk * FBLOCK32, c2off = c1off + FTILE;
+      const int c1n = blk == 0 ? c1off + FBLOCK32 : slot1, c2n = c1n + FTILE;
+      const int c1nn = blk == 0 ? slot1 : slot1 + FBLOCK32;
+      // Hand-scheduled.  dQ / dK: slots 0-15 dP of this block, 16-31 the scores of the next block,
+      // 32-47 the accumulation; dV: 0-15 scores of the next block, 16-31 the accumulation.  LDS
+      // operand f (slots 2f, 2f+1) is requested LA operands earlier into a ring of LA fragments,
+      // across block and step boundaries (both following blocks have landed); the weights of
+      // element pair u are formed in slot WS + WSTEP * u, after dP has drained and before the
       // accumulation needs them.  sched_barrier keeps the compiler from regrouping the slots.
-      auto fetch = [&](int i) {
+      auto fetch = [&](int f) {
         if (MODE == BWD_DV) {
-          if (i < 8) return kread(c1n, i);
-          if (i < 16) return vread(c2off, i - 8);
-          return kread(c1nn, i - 16);
+          if (f < 8) return kread(c1n, f);
+          if (f < 16) return vread(c2off, f - 8);
+          return kread(c1nn, f - 16);
         }
-        if (i < 8) return kread(c2off, i);
-        if (i < 16) return kread(c1n, i - 8);
-        if (i < 24) return vread(c1off, i - 16);
-        return kread(c2n, i - 24);
+        if (f < 8) return kread(c2off, f);
+        if (f < 16) return kread(c1n, f - 8);
+        if (f < 24) return vread(c1off, f - 16);
+        return kread(c2n, f - 24);
       };
       if (!have) {  // first block of a run: nothing was prepared by a previous block
-        s_cur = scores(c1off);
+        scores(c1off, s_cur);
 #pragma unroll
         for (int i = 0; i < LA; ++i) fr[i] = fetch(i);
       }
-      const float* sc = reinterpret_cast<const float*>(smem + slot0 + 2 * TILE_BYTES) + 32 * blk + 4 * h32;
+      const float* sc = reinterpret_cast<const float*>(smem + slot0 + 2 * FTILE) + 32 * blk + 4 * g4;
       if (masked) {  // scores of invisible pairs become -inf (for a positive scale): weight 0
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const bool vis = RMAP::kBlockPredicate ? lane_sees
-                                                 : key_visible(sb_lo + 8 * (e >> 2) + 4 * h32 + (e & 3), kpre, lo_l, hi_l);
-          if (!vis) s_cur[e] = s_hidden;
-        }
+        for (int ct = 0; ct < 2; ++ct)
+#pragma unroll
+          for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const bool vis = RMAP::kBlockPredicate ? lane_sees[rt]
+                                                     : key_visible(sb_lo + 16 * ct + 4 * g4 + e, kpre, lo_l[rt], hi_l[rt]);
+              if (!vis) s_cur[ct][rt][e] = s_hidden;
+            }
       }
-      floatx16 dp, s_next;
+      floatx4 dp[2][2], s_next[2][2];
       bf16x8 wp[2];
-      floatx4 l4[4], d4[4];
-      auto stage = [&](int u) {  // weights of elements 2u, 2u+1: P, or dS = P * (dP - D)
+      floatx4 l4[2], d4[2];  // column scalars of the lane's columns, per column tile
+      // weights of pair u = 4 * rt + 2 * ct + h (columns 16 * ct + 4 * g4 + 2 * h, + 1 of row tile rt): P, or dS = P * (dP - D)
+      auto stage = [&](int u) {
+        const int rt = u >> 2, ct = (u >> 1) & 1, h = u & 1;
         float w[2];
 #pragma unroll
         for (int v = 0; v < 2; ++v) {
-          const int e = 2 * u + v;
-          const float l = ROWS_ARE_QUERIES ? L2_row : l4[e >> 2][e & 3];
-          float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[e], c2, -l));
-          if (MODE != BWD_DV) x *= dp[e] - (ROWS_ARE_QUERIES ? D_row : d4[e >> 2][e & 3]);
+          const int e = 2 * h + v;
+          const float l = ROWS_ARE_QUERIES ? L2_row[rt] : l4[ct][e];
+          float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][rt][e], c2, -l));
+          if (MODE != BWD_DV) x *= dp[ct][rt][e] - (ROWS_ARE_QUERIES ? D_row[rt] : d4[ct][e]);
           w[v] = x;
         }
-        floatx2 f = {w[0], w[1]};
-        bf16x2 h = __builtin_convertvector(f, bf16x2);
-        wp[u >> 2][2 * (u & 3)] = h[0];
-        wp[u >> 2][2 * (u & 3) + 1] = h[1];
+        floatx2 f2 = {w[0], w[1]};
+        bf16x2 h2 = __builtin_convertvector(f2, bf16x2);
+        wp[rt][4 * ct + 2 * h] = h2[0];
+        wp[rt][4 * ct + 2 * h + 1] = h2[1];
       };
+      constexpr int NSLOT = 2 * NFRAG;
 #pragma unroll
       for (int i = 0; i < NSLOT; ++i) {
-        const bf16x8 a = fr[i % LA];
+        const int f = i >> 1, rt = i & 1;
+        const bf16x8 a = fr[f % LA];
         if (MODE == BWD_DV) {
-          if (i < 8) s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, r1f[i], i == 0 ? zero16() : s_next, 0, 0, 0);
-          else acc[(i - 8) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, wp[(i - 8) >> 2], acc[(i - 8) & 3], 0, 0, 0);
+          if (f < 8) s_next[f & 1][rt] = mfma(a, r1f[rt][f >> 1], f < 2 ? zero4 : s_next[f & 1][rt]);
+          else acc[f - 8][rt] = mfma(a, wp[rt], acc[f - 8][rt]);
         } else {
-          if (i < 8) dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, r2f[i], i == 0 ? zero16() : dp, 0, 0, 0);
-          else if (i < 16) s_next = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, r1f[i - 8], i == 8 ? zero16() : s_next, 0, 0, 0);
-          else acc[(i - 16) & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, wp[(i - 16) >> 2], acc[(i - 16) & 3], 0, 0, 0);
+          if (f < 8) dp[f & 1][rt] = mfma(a, r2f[rt][f >> 1], f < 2 ? zero4 : dp[f & 1][rt]);
+          else if (f < 16) s_next[f & 1][rt] = mfma(a, r1f[rt][(f - 8) >> 1], f < 10 ? zero4 : s_next[f & 1][rt]);
+          else acc[f - 16][rt] = mfma(a, wp[rt], acc[f - 16][rt]);
         }
-        fr[i % LA] = fetch(i + LA);
-        if (!ROWS_ARE_QUERIES && i >= W0 - 2 && i < W0 + 6 && ((i - (W0 - 2)) & 1) == 0) {
-          const int t4 = (i - (W0 - 2)) >> 1;  // column scalars of elements 4*t4 .. 4*t4+3, two slots ahead
-          l4[t4] = *reinterpret_cast<const floatx4*>(sc + 8 * t4);
-          if (MODE == BWD_DK) d4[t4] = *reinterpret_cast<const floatx4*>(sc + 64 + 8 * t4);
+        if (rt == 1) fr[f % LA] = fetch(f + LA);
+        if (!ROWS_ARE_QUERIES) {  // column scalars, four slots ahead of the first weight stage
+          if (i == WS - 4) l4[0] = *reinterpret_cast<const floatx4*>(sc);
+          if (i == WS - 3) l4[1] = *reinterpret_cast<const floatx4*>(sc + 16);
+          if (MODE == BWD_DK && i == WS - 2) d4[0] = *reinterpret_cast<const floatx4*>(sc + 64);
+          if (MODE == BWD_DK && i == WS - 1) d4[1] = *reinterpret_cast<const floatx4*>(sc + 64 + 16);
         }
-        if (i >= W0 && i < W0 + 8) stage(i - W0);
+        if (i >= WS && (i - WS) % WSTEP == 0 && (i - WS) / WSTEP < 8) stage((i - WS) / WSTEP);
         __builtin_amdgcn_sched_barrier(0);
       }
-      s_cur = s_next;
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) s_cur[t4 >> 1][t4 & 1] = s_next[t4 >> 1][t4 & 1];
       have = true;
     }
     if (t + 2 < n_steps) put_scalars(slot2);
@@ -412,44 +446,43 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   if (!wave_active) return;
   const float f = MODE == BWD_DV ? 1.f : p.scale;
   if (PARTIAL) {
-    // fp32 partial sums: part[((set * B + batch) * Hkv + kvh) * n_rows + row][128]; lane holds, per
-    // 32 head dims db, the dims 8*(e>>2) + 4*h32 + (e&3) of its row
-    if (row_valid) {
-      float* prow = p.part + ((((int64_t)set * p.B + batch) * p.Hkv + kvh) * n_rows + row) * 128 + 4 * h32;
+    // fp32 partial sums: part[((set * B + batch) * Hkv + kvh) * n_rows + row][128]
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+    for (int rt = 0; rt < 2; ++rt)
+      if (row_valid[rt]) {
+        float* prow = p.part + ((((int64_t)set * p.B + batch) * p.Hkv + kvh) * n_rows + row[rt]) * 128 + 4 * g4;
 #pragma unroll
-        for (int g4 = 0; g4 < 4; ++g4) {
-          floatx4 o4 = {acc[db][4 * g4] * f, acc[db][4 * g4 + 1] * f, acc[db][4 * g4 + 2] * f, acc[db][4 * g4 + 3] * f};
-          *reinterpret_cast<floatx4*>(prow + 32 * db + 8 * g4) = o4;
-        }
-    }
+        for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<floatx4*>(prow + 16 * dt) = acc[dt][rt] * f;
+      }
     return;
   }
-  const bool keep = row_valid && map.store((int)rpos);
-  uint16_t* orow;
-  if (MODE == BWD_DQ) orow = p.dq + (batch * p.dq_bs + rpos * p.dq_rs + hq * p.dq_hs + 8 * h32);
-  else if (MODE == BWD_DK) orow = p.dk + (batch * p.dk_bs + rpos * p.dk_rs + kvh * p.dk_hs + 8 * h32);
-  else orow = p.dv + (batch * p.dv_bs + rpos * p.dv_rs + kvh * p.dv_hs + 8 * h32);
+  // The four lanes of a row hold head dims 4 * g4 .. + 3 of every 16-dim tile; a lane quarter and
+  // its neighbour trade 8 bytes per tile pair so that each lane owns the whole 16-byte chunk
+  // 4 * m + 2 * (g4 % 2) + g4 / 2 of its row.
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int rt = 0; rt < 2; ++rt) {
+    const bool keep = row_valid[rt] && map.store((int)rpos[rt]);
+    uint16_t* orow;
+    const int cofs = (2 * (g4 & 1) + (g4 >> 1)) * 8;
+    if (MODE == BWD_DQ) orow = p.dq + (batch * p.dq_bs + rpos[rt] * p.dq_rs + hq * p.dq_hs + cofs);
+    else if (MODE == BWD_DK) orow = p.dk + (batch * p.dk_bs + rpos[rt] * p.dk_rs + kvh * p.dk_hs + cofs);
+    else orow = p.dv + (batch * p.dv_bs + rpos[rt] * p.dv_rs + kvh * p.dv_hs + cofs);
 #pragma unroll
-    for (int g2 = 0; g2 < 2; ++g2) {
-      uint32_t w[4];
+    for (int m = 0; m < 4; ++m) {
+      uint32_t w[2][2];
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int k2 = 0; k2 < 2; ++k2) {
-          const int e = 8 * g2 + 4 * half + 2 * k2;
-          floatx2 v2 = {acc[db][e] * f, acc[db][e + 1] * f};
-          w[2 * half + k2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
+          floatx2 v2 = {acc[2 * m + t][rt][2 * k2] * f, acc[2 * m + t][rt][2 * k2 + 1] * f};
+          w[t][k2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
         }
-      auto q0 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
-      auto q1 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+      auto q0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
+      auto q1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
       if (keep) {
         u32x4 pk = {q0[0], q1[0], q0[1], q1[1]};
         if (RMAP::kAccumulate) {  // add to what an earlier pass has written (both rounded to bf16)
-          const u32x4 old = *reinterpret_cast<const u32x4*>(orow + 32 * db + 16 * g2);
+          const u32x4 old = *reinterpret_cast<const u32x4*>(orow + 32 * m);
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             floatx2 s2 = {__uint_as_float(pk[i] << 16) + __uint_as_float(old[i] << 16),
@@ -457,9 +490,10 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
             pk[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(s2, bf16x2));
           }
         }
-        *reinterpret_cast<u32x4*>(orow + 32 * db + 16 * g2) = pk;
+        *reinterpret_cast<u32x4*>(orow + 32 * m) = pk;
       }
     }
+  }
 }
 
 // Adds up the partial sums of the sink pass over the chunks and writes the sink rows of dk or dv:

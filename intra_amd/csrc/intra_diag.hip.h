@@ -1,8 +1,8 @@
 // Measurement kernel: what the matrix cores of the board sustain when they do nothing else.
 //
 // Every wavefront of every workgroup (8 per CU) issues back-to-back bf16 MFMAs into independent
-// accumulators, v_mfma_f32_16x16x32_bf16 (SHAPE16: the forward kernel's instruction, 8 accumulators)
-// or v_mfma_f32_32x32x16_bf16 (the backward kernels', 4 accumulators), the same flop count per
+// accumulators, v_mfma_f32_16x16x32_bf16 (SHAPE16: the instruction of the forward and backward kernels, 8 accumulators)
+// or v_mfma_f32_32x32x16_bf16 (the shape these kernels used before, 4 accumulators), the same flop count per
 // iteration either way, on operands taken once from a caller-filled table, so the same launch can
 // be timed with constant and with random operand bits: on a power-limited board the sustained
 // clock, and with it the attainable fraction of the nominal peak, depends on how many operand and
