@@ -46,7 +46,7 @@ int make_request(int domain, int pattern, int B, int S, int H, int Hkv, int arg0
   r->S = S;
   r->H = H;
   r->Hkv = Hkv;
-  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1, 64, 0, 0};  // derived fields: geom_finish() in shape_for()
+  r->geom = IntraGeom{S, 1, 64, 16, 8, 0, 1, 1, 64, 0, 0};  // derived fields: geom_finish() in shape_for()
   r->geom.sink_chunk = 1024;  // backward: set by leading_chunk() once the number of leading keys is known
   if (domain == 0) {
     if (!extended && (pattern == INTRA_LLM_BLOCK_SCATTER || pattern == INTRA_LLM_WINDOW_SINK))
@@ -120,7 +120,22 @@ int default_hp(int ratio) { return ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1)
 
 // Every pattern is one launch of 8-wavefront workgroups.  Image gather0 runs its grid queries as
 // sets of `pg` neighbouring 8x8 patches (as many as fit into a row block) and its text queries -
-// which see what the scatter pattern shows them - as text-only scatter sets of the same launch.
+// which see what the scatter pattern shows them - as sets of the same launch, the text chunks of
+// one or two scatter groups each (MapImgTextRows, pick_text_merge).
+// Text chunks per set of text rows of image gather0 (IntraGeom::tm).  Two chunks in one row block
+// share the text key tiles, but the item then walks through the grid keys of both groups with a
+// quarter of the wavefronts busy, and the static dealing of work items wants items of about one
+// size: 2 if the estimated cost stays within 15 % of a patch item's, else 1.  A key tile with w of
+// 8 wavefronts busy is taken to cost 5/9 + w/18 of a full one (2/3 at w = 2, measured).
+int pick_text_merge(const IntraGeom& ge, int pos, int pg) {
+  const int chunk = ge.text_len / 8, nimg = ge.width * ge.width / 8;
+  if (chunk % 32 != 0 || 2 * chunk > pos) return 1;  // (more chunks than a row block holds share nothing)
+  auto busy = [](int w) { return 5.0 / 9 + std::min(w, 8) / 18.0; };
+  const double patch_item = (ge.text_len + 16 * (16 + 8 * (pg - 1))) / 64.0;
+  const double cost = ge.text_len / 64.0 * busy(2 * chunk / 32) + 2 * (nimg / 64.0) * busy(chunk / 32);
+  return cost <= 1.15 * patch_item ? 2 : 1;
+}
+
 bool shape_for(const Request& r, int hp, Shape* ph) {  // false: no kernel shape fits
   ph->geom = r.geom;
   ph->hp = hp;
@@ -142,6 +157,7 @@ bool shape_for(const Request& r, int hp, Shape* ph) {  // false: no kernel shape
       while (np % pg != 0) --pg;
       ph->map = MAP_IMG_GATHER0;
       ph->geom.pg = pg;
+      ph->geom.tm = pick_text_merge(r.geom, 8 * 32 / hp, pg);
     }
   }
   geom_finish(ph->geom);
@@ -191,7 +207,7 @@ auto by_map(int map, A&&... a) {
     case MAP_IMG_SCATTER: return F<MapImgScatter>::go(a...);
     case MAP_LLM_BLOCK_SCATTER: return F<MapLlmBlockScatter>::go(a...);
     case MAP_LLM_WINDOW_SINK: return F<MapLlmWindowSink>::go(a...);
-    default: return F<MapImgGather0>::go(a...);
+    default: return F<MapImgGather0F>::go(a...);
   }
 }
 template <class MAP> struct DimsOf { static LaunchDims go(const Request& r, const Shape& ph) { return dims_of<MAP>(r, ph); } };
@@ -337,12 +353,14 @@ bool use_fast_softmax(float scale) {
   return fabsf(scale) <= INTRA_FAST_SOFTMAX_MAX_SCALE;
 }
 
-// Order of an XCD's work items (see KParams::Section).  One section - every pair, all row blocks - except
-// where a launch mixes full-size items with items that keep only a quarter of the workgroup busy:
+// Order of an XCD's work items (see KParams::Section).  One section - every pair, all row blocks -
+// except where a launch mixes kinds of items:
 //  * image scatter: a set has text_len / 8 + width^2 / 8 queries, so its last row block is partial
-//    (64 of 256 rows at 24 heads); those row blocks of all pairs form a second section;
-//  * image gather0: the text-only sets (64 queries each, against text + one group's grid keys) and
-//    the patch runs (256 queries against text + window keys); whichever kind takes longer goes first.
+//    (64 of 256 rows at 24 heads); where it is at most half full, those row blocks of all pairs
+//    form a second section behind the full ones;
+//  * image gather0: the text rows (the first sets; pairs are numbered set-major, so they are the
+//    first pair slots) and the patch runs can have different numbers of row blocks; each kind gets
+//    its section, so that no number goes to an empty item, text rows first.
 void set_sections(intra::KParams& p, const Request& r, const Shape& ph, const LaunchDims& d) {
   const int pslots = (d.n_pairs + 7) / 8;
   auto section = [&](int p_lo, int p_n, int mb_lo, int mb_hi) {
@@ -362,15 +380,14 @@ void set_sections(intra::KParams& p, const Request& r, const Shape& ph, const La
       p.sec[1] = section(0, pslots, d.n_mblocks - 1, d.n_mblocks);
     }
   } else if (ph.map == MAP_IMG_GATHER0) {
-    // pairs are numbered set-major, so the 8 text sets are the pair slots below B * Hkv
-    const int text_slots = r.B * r.Hkv;
-    const int64_t text_keys = r.geom.text_len + (int64_t)r.geom.width * r.geom.width / 8;
-    const int64_t patch_keys = r.geom.text_len + 16 * (16 + 8 * (ph.geom.pg - 1));
-    // a text item keeps 2 of 8 wavefronts busy and runs a key tile in about 2/3 of the time
-    if (3 * patch_keys > 2 * text_keys && pslots > text_slots) {
-      p.sec[0] = section(text_slots, pslots - text_slots, 0, d.n_mblocks);
-      p.sec[1] = section(0, text_slots, 0, d.n_mblocks);
-    }
+    // pair slots that hold text rows only (a slot mixing both kinds goes with the patch runs and
+    // then keeps the larger number of row blocks)
+    const int text_pairs = (8 / ph.geom.tm) * r.B * r.Hkv;
+    const int text_slots = text_pairs / 8;
+    const int text_mb = std::min(d.n_mblocks, (ph.geom.tm * (r.geom.text_len / 8) + d.pos - 1) / d.pos);
+    const int patch_mb = text_pairs % 8 != 0 ? d.n_mblocks : std::min(d.n_mblocks, (64 * ph.geom.pg + d.pos - 1) / d.pos);
+    p.sec[0] = section(0, text_slots, 0, text_mb);
+    p.sec[1] = section(text_slots, pslots - text_slots, 0, patch_mb);
   }
   p.n_slots = p.sec[0].slots + p.sec[1].slots;
 }

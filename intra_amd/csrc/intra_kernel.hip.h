@@ -87,8 +87,9 @@ struct KParams {
   int n_pairs;         // B * Hkv * n_sets
   int n_slots;         // work items per XCD: sum of the sections' slots
   // The work items of an XCD are numbered section by section (costly kinds of items first, so
-  // that the cheap ones fill the last, partial round of the workgroups): a section is a range of
-  // the XCD's pairs times a range of row blocks, taken pair by pair, last row block first.
+  // that the cheap ones fill the last, partial round of the workgroups; kinds of sets with
+  // different numbers of row blocks apart, so that no number goes to an empty item): a section is
+  // a range of the XCD's pairs times a range of row blocks, taken pair by pair, last row block first.
   struct Section {
     int p_lo;          // first pair slot (pair = 8 * pair slot + XCD)
     int mb_hi;         // one past its last row block

@@ -76,6 +76,7 @@ struct IntraGeom {
   int text_len;  // image: text tokens in front of the grid
   int text_only; // image scatter: only the text queries of each group (the text rows of gather0)
   int pg;        // image gather0: 8x8 patches per set (a run of pg patches in one patch row)
+  int tm;        // image gather0, forward: text chunks (scatter groups) per set of text rows: 1 or 2
   int blk;       // LLM block scatter: tokens per block
   int off;       // LLM block scatter: stripe offset, 0 <= off < G
   int ns;        // LLM block scatter / window with sinks: leading tokens every query sees
@@ -267,6 +268,75 @@ struct MapImgGather0 {
   IM_HD int kpos(int t) const { return is_text ? sc.kpos(t) : pa.kpos(t); }
   IM_HD int klo(int tq) const { return is_text ? 0 : pa.klo(tq); }
   IM_HD int khi(int tq) const { return is_text ? sc.khi(tq) : pa.khi(tq); }
+};
+
+// ---- The forward launch of image gather0 deals the text queries like this.  A scatter group has
+// only text_len / 8 text queries (64 at 512 text tokens), a quarter of a row block, and they see
+// the text keys and the group's grid keys; so the text chunks of tm = 1 or 2 groups share one row
+// block (8 / tm sets of text rows per head).  With two groups A, B the key list is
+// [grid keys of A][text keys][grid keys of B]: the queries of A see the first two parts, those of
+// B the last two, each a contiguous range, and the text key tiles are loaded once for both.  A
+// row block that holds one group's chunk only has the list [text keys][grid keys] of a scatter
+// set.  (Image scatter keeps its text queries in front of the grid queries of their group,
+// MapImgScatter: its key bounds are compile-time constants that way, which its main loop needs.)
+struct MapImgTextRows {
+  static constexpr bool kHasPrefix = false;
+  IM_HD int kpre() const { return 0; }
+  // (few fields: two of these maps are live in the kernel's main loop, in scalar registers)
+  int W, T, nimg, nq_, lead, cA, cB, q0;
+  FastDiv dWq;
+  static IM_HD int num_sets(const IntraGeom& ge) { return 8 / ge.tm; }
+  static IM_HD int max_nq(const IntraGeom& ge) { return ge.tm * (ge.text_len / 8); }
+  IM_HD MapImgTextRows(const IntraGeom& ge, int set, int t0) {
+    W = ge.width;
+    T = ge.text_len;
+    nimg = W * W / 8;
+    dWq = ge.dWq;
+    const int chunk = T / 8;
+    const int first = ge.tm * set;
+    const int g0 = ge.tm == 2 && t0 >= chunk ? 1 : 0;  // chunk of the row block's first query
+    const int gA = first + g0;
+    nq_ = ge.tm * chunk;
+    q0 = first * chunk;
+    lead = ge.tm - g0 == 2 ? nimg : 0;     // two groups: the grid keys of the first in front of the text keys
+    cA = T + (gA >> 2) * W + (gA & 3);     // position of grid token 0 of group gA
+    cB = cA + (lead ? 1 : 0);              // ... of the group whose grid keys follow the text keys
+  }
+  // Grid token u of scatter group g sits at row g / 4 + 2 * (u / (W/4)), column g % 4 + 4 * (u % (W/4)):
+  // position T + (g / 4) * W + g % 4 + 4 * u + (u / (W/4)) * W.  Groups gA and gA + 1 of a two-group
+  // list differ by one column.
+  IM_HD int grid(int c0, int u) const { return c0 + 4 * u + (int)fd_div(u, dWq) * W; }
+  IM_HD int nq() const { return nq_; }
+  IM_HD int nk() const { return T + lead + nimg; }
+  IM_HD int qpos(int t) const { return q0 + t; }
+  IM_HD int kpos(int t) const {  // (runs per fetched key row: two compares, no mask arithmetic)
+    const unsigned tt = (unsigned)(t - lead);  // index behind the leading part (huge inside it): text, then grid
+    const bool front = t < lead;
+    const int p = grid(front ? cA : cB, front ? t : (int)tt - T);
+    return tt < (unsigned)T ? (int)tt : p;
+  }
+  // with two groups the queries of the second chunk start behind the first group's grid keys
+  IM_HD int klo(int tq) const { return 8 * tq >= T ? lead : 0; }
+  IM_HD int khi(int tq) const { return klo(tq) + T + nimg - 1; }
+};
+
+// image gather0, forward launch: the text rows, then the patch runs
+struct MapImgGather0F {
+  static constexpr bool kHasPrefix = true;
+  bool is_text;
+  MapImgTextRows tx;
+  MapImgPatch pa;
+  static IM_HD int num_sets(const IntraGeom& ge) { return MapImgTextRows::num_sets(ge) + MapImgPatch::num_sets(ge); }
+  static IM_HD int max_nq(const IntraGeom& ge) { return im_max(MapImgTextRows::max_nq(ge), MapImgPatch::max_nq(ge)); }
+  IM_HD MapImgGather0F(const IntraGeom& ge, int set, int t0)
+      : is_text(set < 8 / ge.tm), tx(ge, is_text ? set : 0, t0), pa(ge, is_text ? 0 : set - 8 / ge.tm, t0) {}
+  IM_HD int nq() const { return is_text ? tx.nq() : pa.nq(); }
+  IM_HD int nk() const { return is_text ? tx.nk() : pa.nk(); }
+  IM_HD int kpre() const { return is_text ? 0 : pa.kpre(); }
+  IM_HD int qpos(int t) const { return is_text ? tx.qpos(t) : pa.qpos(t); }
+  IM_HD int kpos(int t) const { return is_text ? tx.kpos(t) : pa.kpos(t); }
+  IM_HD int klo(int tq) const { return is_text ? tx.klo(tq) : pa.klo(tq); }
+  IM_HD int khi(int tq) const { return is_text ? tx.khi(tq) : pa.khi(tq); }
 };
 
 // ------- LLM block scatter: blocks of blk tokens, block b in group b % G.  A query of block qb sees,

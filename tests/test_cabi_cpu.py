@@ -39,13 +39,19 @@ def test_plan_headline(lib):
 
 
 def test_plan_gather0_sets(lib):
-    # one launch: 8 text-only scatter sets, then sets of 4 / 2 / 1 neighbouring 8x8 patches
+    # one launch: sets of text rows (the 64 text queries of 1 or 2 scatter groups each), then sets of
+    # 4 / 2 / 1 neighbouring 8x8 patches.  At 2048 x 2048 a merged text item would be much longer than
+    # a patch item, so the chunks stay apart; at 1024 x 1024 two share a row block.
     for H, Hkv, hp, pg in ((24, 24, 1, 4), (16, 8, 2, 2), (32, 8, 4, 1)):
         rc, p = _plan(lib, 1, 4, 1, 16896, H, Hkv, 128, 512)
         assert rc == 0 and p.launches == 1
         assert (p.heads_per_block, p.waves, p.pos_per_block) == (hp, 8, 256 // hp)
         assert (p.n_sets, p.n_mblocks) == (8 + 16 * 16 // pg, 1)
         assert p.work_items == 8 * -(-Hkv * p.n_sets // 8) * (H // Hkv // hp)
+    rc, p = _plan(lib, 1, 4, 1, 4608, 24, 24, 64, 512)
+    assert rc == 0 and (p.n_sets, p.n_mblocks) == (4 + 8 * 8 // 4, 1)
+    rc, p = _plan(lib, 1, 0, 1, 4608, 24, 24, 64, 512)
+    assert rc == 0 and (p.n_sets, p.n_mblocks) == (8, 3)
     rc, p = _plan(lib, 1, 0, 1, 16896, 24, 24, 128, 512)
     assert rc == 0 and p.launches == 1
 
