@@ -389,7 +389,10 @@ def test_random_llm_shapes(case):
     assert bool(((lse - ref).abs() <= LSE_ATOL + 2e-3 * ref.abs()).all())
 
 
-@pytest.mark.parametrize("width,text_len,H,Hkv", [(24, 72, 4, 4), (40, 8, 8, 2), (16, 200, 2, 1), (32, 96, 4, 1)])
+# (the last three: text chunks of 32 / 64 queries, where gather0 puts the chunks of two scatter groups into
+# one row block, on grids whose groups are not multiples of a key tile, and with grouped query heads)
+@pytest.mark.parametrize("width,text_len,H,Hkv", [(24, 72, 4, 4), (40, 8, 8, 2), (16, 200, 2, 1), (32, 96, 4, 1),
+                                                  (32, 256, 4, 4), (48, 512, 3, 3), (40, 512, 4, 2)])
 @pytest.mark.parametrize("pattern,pid", [("scatter", 0), ("gather0", 4)])
 def test_image_other_text_lengths_through_the_c_abi(width, text_len, H, Hkv, pattern, pid):
     """The Python entry point fixes 512 text tokens like the reference; the C ABI takes any multiple
