@@ -44,7 +44,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--seqlen", type=int, default=32768)
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--softmax", choices=["auto", "exact", "fast"], default="auto",
+    ap.add_argument("--softmax", choices=["auto", "exact", "scaled", "folded"], default="auto",
                     help="softmax arithmetic of the kernel (auto: what a plain call gets)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run three plain 1 GiB device copies, the known-size kernel that scales "

@@ -5,8 +5,11 @@
  * arguments are raw device pointers to bf16 data laid out (batch, token, head, 128) with the
  * last dimension contiguous; strides are passed in ELEMENTS as {batch, token, head}.  Every
  * pointer and every stride must keep 16-byte alignment (pointer % 16 == 0, stride % 8 == 0).
- * The library allocates nothing and keeps no state between calls; the caller owns `o`.
- * Launches are asynchronous on `hip_stream` (a hipStream_t, NULL = default stream).
+ * The library allocates nothing; the caller owns `o`.  Launches are asynchronous on `hip_stream`
+ * (a hipStream_t, NULL = default stream).  State the library keeps between calls: the process
+ * default of the softmax arithmetic (intra_set_softmax_mode; a call can name its own in the flags
+ * of the *_ex entry points), the 16 MiB per-GPU array behind intra_llm_bwd_noalloc, the timer buffer
+ * of measurement builds (intra_diag_set_buffer), and per-device caches of the CU count.
  *
  * Every function returns INTRA_OK or an error code; intra_last_error() then describes the failure
  * (thread-local string).  Argument validation happens before any HIP call, so it can be exercised
@@ -89,33 +92,54 @@ int intra_image_fwd_lse(const void* q, const void* k, const void* v, void* o, in
  *     or (offset != 0 and kb == qb).  0 <= offset < group_num, 0 <= n_sink <= block.  With
  *     offset != 0, block must be a multiple of 256 / min(4, largest power of two in H / Hkv).
  *   INTRA_LLM_WINDOW_SINK: query i sees key j <= i iff i - j < window or j < n_sink
- *     (window >= 1, n_sink >= 0; group_num ignored). */
+ *     (window >= 1, n_sink >= 0; group_num ignored).
+ *   flags: INTRA_SOFTMAX_* (below) for this call; other bits must be 0. */
 int intra_llm_fwd_ex(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
                      int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
                      const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
                      int group_num, int window, int block, int offset, int n_sink,
-                     float softmax_scale, void* hip_stream, float* lse, const int64_t lse_strides[3]);
+                     float softmax_scale, void* hip_stream, float* lse, const int64_t lse_strides[3],
+                     unsigned flags);
+/* intra_image_fwd with an optional log-sum-exp output (lse may be NULL) and per-call flags. */
+int intra_image_fwd_ex(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                       int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                       const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                       int width, int text_len, float softmax_scale, void* hip_stream, float* lse,
+                       const int64_t lse_strides[3], unsigned flags);
 
 /* Description of the last failure on the calling thread ("" if none).  Replaces the
  * TORCH_CHECK messages of flash_api.cpp. */
 const char* intra_last_error(void);
 
-/* Library version, major*10000 + minor*100 + patch (0.2.0). */
-#define INTRA_VERSION 200
+/* Library version, major*10000 + minor*100 + patch (0.3.0). */
+#define INTRA_VERSION 300
 int intra_version(void);
 
 /* Softmax arithmetic of the forward entry points.  The reference scales the fp32 scores after the
- * first product (csrc/flash_attn/src/softmax.h:65-91); so does the EXACT mode here.  FAST multiplies
- * softmax_scale * log2(e) into the bf16 query rows instead and forms the weights without a running
- * maximum; queries whose weight sum leaves 2^-100 .. 2^60 are recomputed in EXACT arithmetic inside
- * the same launch, so results stay finite and correct for any input.  FAST perturbs a score of s
- * nats by about 1.1e-3 * |s| nats rms (bf16 rounding of the scaled query), beside the 1.1e-3
- * relative rms that rounding a weight to bf16 costs in both modes.
- *   mode 0 (default): FAST iff |softmax_scale| <= INTRA_FAST_SOFTMAX_MAX_SCALE (twice 128^-1/2)
- *   mode 1: always EXACT        mode 2: always FAST
- * The setting is process-wide and starts from the environment variable INTRA_SOFTMAX
- * (auto / exact / fast).  No counterpart in the reference. */
-#define INTRA_FAST_SOFTMAX_MAX_SCALE 0.1767767f
+ * first product and subtracts a running maximum (csrc/flash_attn/src/softmax.h:65-91).
+ *   INTRA_SOFTMAX_EXACT:  that arithmetic (the running reference only moves when a block maximum
+ *       leaves +-60 powers of two, which changes no result).
+ *   INTRA_SOFTMAX_SCALED: the same fp32 scaling, weights exp2(score * scale * log2 e) with no
+ *       running maximum; queries whose weight sum leaves 2^-100 .. 2^60 are recomputed in EXACT
+ *       arithmetic inside the same launch, so results stay finite and correct for any input.  Equal
+ *       to EXACT up to the rounding of the weights; accuracy does not depend on the size of q, k.
+ *   INTRA_SOFTMAX_FOLDED: multiplies softmax_scale * log2(e) into the bf16 query rows instead (one
+ *       multiply per score less; about 2 % faster), then as SCALED.  Rounding the scaled query to
+ *       bf16 perturbs a score by about 1.1e-3 * scale * sqrt(sum_d q_d^2 k_d^2) rms, i.e. in
+ *       proportion to the magnitudes of q and k: as accurate as the other two for unit-variance
+ *       inputs, outside the 1.6e-2 output bound once q and k are about twice as large.  Opt-in.
+ *   INTRA_SOFTMAX_AUTO (0): the process default, which starts as "SCALED iff |softmax_scale| <=
+ *       INTRA_SCALED_SOFTMAX_MAX_SCALE (four times 128^-1/2), else EXACT".
+ * A call names its arithmetic in the `flags` of intra_llm_fwd_ex / intra_image_fwd_ex; the entry
+ * points without flags use the process default.  intra_set_softmax_mode changes that default for
+ * the whole process (it starts from the environment variable INTRA_SOFTMAX: auto / exact / folded
+ * / scaled); it is meant for experiments - callers that need a fixed arithmetic pass it per call.
+ * No counterpart in the reference. */
+enum {
+  INTRA_SOFTMAX_AUTO = 0, INTRA_SOFTMAX_EXACT = 1, INTRA_SOFTMAX_FOLDED = 2, INTRA_SOFTMAX_SCALED = 3,
+  INTRA_SOFTMAX_MASK = 3
+};
+#define INTRA_SCALED_SOFTMAX_MAX_SCALE 0.35355339f
 int intra_set_softmax_mode(int mode);
 int intra_get_softmax_mode(void);
 

@@ -11,4 +11,4 @@ except ImportError as _err:
     intra_llm_attn = intra_llm_attn_bwd = intra_llm_attn_func = _missing
     get_softmax_mode = set_softmax_mode = _missing
 
-__version__ = "0.2.0"  # intra_version() of the library: 200
+__version__ = "0.3.0"  # intra_version() of the library: 300

@@ -30,7 +30,8 @@ SYMBOLS = {
     "intra_image_fwd_lse": (ctypes.c_int, _FWD_ARGS + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64)]),
     "intra_llm_fwd_ex": (ctypes.c_int, [ctypes.c_void_p] * 4 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 4 +
                          [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_void_p,
-                                               ctypes.POINTER(ctypes.c_int64)]),
+                                               ctypes.POINTER(ctypes.c_int64), ctypes.c_uint]),
+    "intra_image_fwd_ex": (ctypes.c_int, _FWD_ARGS + [ctypes.c_void_p, ctypes.POINTER(ctypes.c_int64), ctypes.c_uint]),
     "intra_llm_bwd": (ctypes.c_int, [ctypes.c_void_p] * 10 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 9 +
                       [ctypes.c_int] * 6 + [ctypes.c_float, ctypes.c_void_p]),
     "intra_llm_bwd_noalloc": (ctypes.c_int, [ctypes.c_void_p] * 9 + [ctypes.c_int] * 4 + [ctypes.POINTER(ctypes.c_int64)] * 9 +

@@ -304,22 +304,31 @@ int launch_grid(int work_items) {
   return work_items < g ? work_items : g;
 }
 
-template <class MAP, int HP, int NW, bool FAST>
+template <class MAP, int HP, int NW, int SM>
 int launch(const intra::KParams& p, int grid, hipStream_t stream) {
-  hipLaunchKernelGGL((intra::intra_fwd_kernel<MAP, HP, NW, FAST>), dim3(grid), dim3(NW * 64), 0, stream, p);
+  hipLaunchKernelGGL((intra::intra_fwd_kernel<MAP, HP, NW, SM>), dim3(grid), dim3(NW * 64), 0, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
   return INTRA_OK;
 }
 
+template <class MAP, int HP>
+int launch_sm(const intra::KParams& p, int sm, int grid, hipStream_t stream) {
+  switch (sm) {
+    case intra::SM_SCALED: return launch<MAP, HP, 8, intra::SM_SCALED>(p, grid, stream);
+    case intra::SM_FOLDED: return launch<MAP, HP, 8, intra::SM_FOLDED>(p, grid, stream);
+    default: return launch<MAP, HP, 8, intra::SM_EXACT>(p, grid, stream);
+  }
+}
+
 template <class MAP>
 struct LaunchMap {
-  static int go(const intra::KParams& p, int hp, int nw, bool fast, int grid, hipStream_t stream) {
+  static int go(const intra::KParams& p, int hp, int nw, int sm, int grid, hipStream_t stream) {
     if (nw == 8) {
       switch (hp) {
-        case 4: return fast ? launch<MAP, 4, 8, true>(p, grid, stream) : launch<MAP, 4, 8, false>(p, grid, stream);
-        case 2: return fast ? launch<MAP, 2, 8, true>(p, grid, stream) : launch<MAP, 2, 8, false>(p, grid, stream);
-        case 1: return fast ? launch<MAP, 1, 8, true>(p, grid, stream) : launch<MAP, 1, 8, false>(p, grid, stream);
+        case 4: return launch_sm<MAP, 4>(p, sm, grid, stream);
+        case 2: return launch_sm<MAP, 2>(p, sm, grid, stream);
+        case 1: return launch_sm<MAP, 1>(p, sm, grid, stream);
       }
     }
     return fail(INTRA_ERR_UNSUPPORTED, "no kernel for heads_per_block=%d, waves=%d", hp, nw);
@@ -330,27 +339,36 @@ struct LaunchMap {
 std::atomic<long long*> g_diag{nullptr};
 std::atomic<int64_t> g_diag_values{0};
 
-// Softmax arithmetic of the forward kernels: 0 = by softmax_scale (see use_fast_softmax), 1 = always
-// EXACT, 2 = always FAST.  Starts from the environment variable INTRA_SOFTMAX (auto / exact / fast).
+// What a call that names no softmax arithmetic gets (INTRA_SOFTMAX_* values; 0 = by softmax_scale,
+// see pick_softmax).  Starts from the environment variable INTRA_SOFTMAX (auto / exact / folded /
+// scaled; "fast" is the older name of folded).
 std::atomic<int>& softmax_mode() {
   static std::atomic<int> mode{[] {
     const char* e = getenv("INTRA_SOFTMAX");
-    if (e && !strcmp(e, "exact")) return 1;
-    if (e && !strcmp(e, "fast")) return 2;
-    return 0;
+    if (e && !strcmp(e, "exact")) return (int)INTRA_SOFTMAX_EXACT;
+    if (e && (!strcmp(e, "folded") || !strcmp(e, "fast"))) return (int)INTRA_SOFTMAX_FOLDED;
+    if (e && !strcmp(e, "scaled")) return (int)INTRA_SOFTMAX_SCALED;
+    return (int)INTRA_SOFTMAX_AUTO;
   }()};
   return mode;
 }
 
-// FAST rounds Q * softmax_scale * log2(e) to bf16 before the MFMA.  That perturbs a score of s nats
-// by about 2^-9 * |s| / sqrt(3) nats rms (every product q_d * k_d moves by up to 2^-9 of itself),
-// against the 2^-9 / sqrt(3) relative rms that rounding the weight to bf16 costs in either mode.
-// Up to twice the default scale d^-1/2 the scores of unit-variance inputs are a few nats and the
-// two are of one size; beyond that the fp32 scaling of the reference's arithmetic is kept.
-bool use_fast_softmax(float scale) {
-  const int mode = softmax_mode().load(std::memory_order_relaxed);
-  if (mode != 0) return mode == 2;
-  return fabsf(scale) <= INTRA_FAST_SOFTMAX_MAX_SCALE;
+// The kernel's softmax arithmetic for a call: what its flags name, else the process default.  Auto
+// takes SCALED - fp32 scores times scale like the reference, no running maximum, out-of-band
+// queries recomputed - while |softmax_scale| <= INTRA_SCALED_SOFTMAX_MAX_SCALE; beyond that the
+// scores of ordinary inputs spread over so many powers of two that most work items would be
+// computed twice, and EXACT runs from the start.  FOLDED is never picked by auto: its error grows
+// with the magnitude of q and k (every product q_d * k_d moves by up to 2^-9 of itself when
+// Q * scale * log2(e) is rounded to bf16).
+int pick_softmax(float scale, unsigned flags) {
+  int mode = (int)(flags & INTRA_SOFTMAX_MASK);
+  if (mode == INTRA_SOFTMAX_AUTO) mode = softmax_mode().load(std::memory_order_relaxed);
+  switch (mode) {
+    case INTRA_SOFTMAX_EXACT: return intra::SM_EXACT;
+    case INTRA_SOFTMAX_FOLDED: return intra::SM_FOLDED;
+    case INTRA_SOFTMAX_SCALED: return intra::SM_SCALED;
+    default: return fabsf(scale) <= INTRA_SCALED_SOFTMAX_MAX_SCALE ? intra::SM_SCALED : intra::SM_EXACT;
+  }
 }
 
 // Order of an XCD's work items (see KParams::Section).  One section - every pair, all row blocks -
@@ -414,8 +432,9 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
         int Hkv, const int64_t* qs, const int64_t* ks, const int64_t* vs, const int64_t* os,
         int pattern, int arg0, int arg1, float scale, void* stream, float* lse = nullptr,
         const int64_t* ls = nullptr, bool want_lse = false, int block = 0, int offset = 0, int n_sink = 0,
-        bool extended = false) {
+        bool extended = false, unsigned flags = 0) {
   g_err[0] = 0;
+  if (flags & ~(unsigned)INTRA_SOFTMAX_MASK) return fail(INTRA_ERR_INVALID, "unknown bits in flags (0x%x)", flags);
   Request r;
   int rc = make_request(domain, pattern, B, S, H, Hkv, arg0, arg1, &r, block, offset, n_sink, extended);
   if (rc) return rc;
@@ -479,7 +498,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.d_hkv = make_fastdiv(Hkv);
   p.d_hgroups = make_fastdiv(p.hgroups);
   p.diag = (int64_t)grid * intra::DIAG_SLOTS <= g_diag_values.load() ? g_diag.load() : nullptr;
-  return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, use_fast_softmax(scale), grid, static_cast<hipStream_t>(stream));
+  return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, pick_softmax(scale, flags), grid, static_cast<hipStream_t>(stream));
 }
 
 
@@ -910,7 +929,8 @@ int intra_version(void) { return INTRA_VERSION; }
 
 int intra_set_softmax_mode(int mode) {
   g_err[0] = 0;
-  if (mode < 0 || mode > 2) return fail(INTRA_ERR_INVALID, "softmax mode must be 0 (auto), 1 (exact) or 2 (fast), got %d", mode);
+  if (mode < 0 || mode > 3)
+    return fail(INTRA_ERR_INVALID, "softmax mode must be 0 (auto), 1 (exact), 2 (folded) or 3 (scaled), got %d", mode);
   softmax_mode().store(mode, std::memory_order_relaxed);
   return INTRA_OK;
 }
@@ -976,10 +996,21 @@ int intra_llm_fwd_ex(const void* q, const void* k, const void* v, void* o, int B
                      int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
                      const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
                      int group_num, int window, int block, int offset, int n_sink,
-                     float softmax_scale, void* hip_stream, float* lse, const int64_t lse_strides[3]) {
+                     float softmax_scale, void* hip_stream, float* lse, const int64_t lse_strides[3],
+                     unsigned flags) {
   return run(0, q, k, v, o, B, S, H, Hkv, q_strides, k_strides, v_strides, o_strides, pattern,
              group_num, window, softmax_scale, hip_stream, lse, lse_strides, lse != nullptr, block, offset,
-             n_sink, true);
+             n_sink, true, flags);
+}
+
+int intra_image_fwd_ex(const void* q, const void* k, const void* v, void* o, int B, int S, int H,
+                       int Hkv, const int64_t q_strides[3], const int64_t k_strides[3],
+                       const int64_t v_strides[3], const int64_t o_strides[3], int pattern,
+                       int width, int text_len, float softmax_scale, void* hip_stream, float* lse,
+                       const int64_t lse_strides[3], unsigned flags) {
+  return run(1, q, k, v, o, B, S, H, Hkv, q_strides, k_strides, v_strides, o_strides, pattern,
+             width, text_len, softmax_scale, hip_stream, lse, lse_strides, lse != nullptr, 0, 0, 0, false,
+             flags);
 }
 
 int intra_plan_llm_ex(int pattern, int B, int S, int H, int Hkv, int group_num, int window,

@@ -38,14 +38,16 @@
 //  * Blocks outside a wavefront's key range are skipped; only blocks cut by a bound are masked.
 //  * The grid is persistent (about one workgroup per CU); work items are dealt per XCD so that
 //    one (batch, kv head, set) stays in one XCD's L2, in an order that balances causal triangles.
-//  * Two softmax modes.  EXACT scales the fp32 scores after the MFMA and watches every block's
-//    maximum (the reference's arithmetic, csrc/flash_attn/src/softmax.h:65-91).  FAST folds
+//  * Three softmax modes.  SM_EXACT scales the fp32 scores after the MFMA and watches every
+//    block's maximum (the reference's arithmetic, csrc/flash_attn/src/softmax.h:65-91).
+//    SM_SCALED (what a plain call gets) scales the fp32 scores the same way, so its accuracy does
+//    not depend on the size of q and k, but keeps no running maximum at all: weights are
+//    exp2(score * c); a query whose weight sum left the safe exponent band marks its work item
+//    in an LDS bitmap, and after the last item the workgroup runs the marked items again in
+//    SM_EXACT mode.  SM_FOLDED (opt-in per call) saves the multiply per score as well: it folds
 //    softmax_scale * log2(e) into the bf16 Q fragments once per work item and exponentiates the
-//    raw MFMA results with no running maximum at all; a query whose weight sum left the safe
-//    exponent band marks its work item in an LDS bitmap, and after the last item the workgroup
-//    runs the marked items again in EXACT mode.  The host picks FAST for |softmax_scale| up to
-//    twice the default (there the bf16 rounding of Q * c adds less noise to a weight than the
-//    bf16 rounding of the weight itself does for scores of a few nats).
+//    raw MFMA results; the bf16 rounding of Q * c perturbs a score in proportion to the
+//    magnitudes of q and k, so it is only as accurate as the other two for inputs of unit scale.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -79,7 +81,7 @@ struct KParams {
   IntraGeom geom;
   float scale_log2;    // |softmax_scale| * log2(e)
   int negate_q;        // softmax_scale < 0: flip the sign of Q instead
-  float q_fold;        // FAST mode: softmax_scale * log2(e), signed, multiplied into Q
+  float q_fold;        // SM_FOLDED: softmax_scale * log2(e), signed, multiplied into Q
   uint32_t k_rs_bytes, v_rs_bytes, q_rs_bytes;  // token strides of k, v, q in bytes (< 4 GiB, checked on the host)
   int n_sets;          // sets per (batch, kv head)
   int n_mblocks;       // row blocks of the largest set
@@ -111,6 +113,9 @@ constexpr int DIAG_SLOTS = 8;
 #else
 #define INTRA_DIAG(...)
 #endif
+
+// softmax arithmetic of a pass (template argument SM)
+constexpr int SM_EXACT = 0, SM_FOLDED = 1, SM_SCALED = 2;
 
 constexpr int BN = 64;             // keys per tile (one barrier per tile)
 // LDS tile layout.  A tile is 16 groups of 4 rows; a group is 1024 contiguous bytes (what one
@@ -175,11 +180,13 @@ __device__ __forceinline__ float lane_quad_sum(float x) {
 template <int V>
 using ic = std::integral_constant<int, V>;
 
-// One pass of a workgroup over its work items.  FAST: see the file comment.  REDO: visit only the
-// items whose round is marked in `redo` (the EXACT second pass of a FAST kernel).
-template <class MAP, int HP, int NW, bool FAST, bool REDO>
+// One pass of a workgroup over its work items.  SM: softmax arithmetic, see the file comment.
+// REDO: visit only the items whose round is marked in `redo` (the SM_EXACT second pass of a kernel
+// whose first pass keeps no running maximum).
+template <class MAP, int HP, int NW, int SM, bool REDO>
 __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, uint32_t* redo) {
   constexpr int POS = NW * 32 / HP;          // in-set queries per row block
+  constexpr bool FAST = SM != SM_EXACT;      // no running maximum: the weight sums are checked at the end
   static_assert(BN % NW == 0, "tile rows must split evenly over the wavefronts");
   static_assert(!(FAST && REDO), "the second pass is exact");
 
@@ -459,7 +466,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) raw[4 * qt + ks] = __builtin_bit_cast(u32x4, kread_q(qa + qt * qstep + 64 * (ks ^ r)));
-    if (FAST) {  // Q <- bf16(Q * softmax_scale * log2 e): the MFMA then yields exponents directly
+    if (SM == SM_FOLDED) {  // Q <- bf16(Q * softmax_scale * log2 e): the MFMA then yields exponents directly
       const float cq = p.q_fold;
 #pragma unroll
       for (int f = 0; f < 8; ++f)
@@ -494,8 +501,8 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   // nothing overflows or underflows.  fp32 and bf16 both span 2^+-126, so mref stays 0 (and costs
   // nothing) for every query whose scores stay within +-60 of it; it is re-centred on a block's
   // maximum when that maximum leaves this band upwards, or downwards before anything was
-  // accumulated.  FAST mode has no reference at all (weights exp2(score), scores already in
-  // exponent units).
+  // accumulated.  SM_SCALED and SM_FOLDED have no reference at all (weights exp2(score * c), or
+  // exp2(score) with the scores already in exponent units).
   float mref[2] = {0.f, 0.f};
   float l_acc[2] = {0.f, 0.f};  // this lane's share of the two queries' weight sums
   const float c = p.scale_log2;  // |softmax_scale| * log2(e)
@@ -597,9 +604,12 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     // pair u = 4 * qt + 2 * kt + h: weights of keys 16 * kt + 4 * g4 + 2 * h, + 1 for query tile qt
     auto stage_e = [&](int u) {
       const int qt = u >> 2, kt = (u >> 1) & 1, h = u & 1;
-      if (FAST) {
+      if (SM == SM_FOLDED) {
         px[u][0] = __builtin_amdgcn_exp2f(s[kt][qt][2 * h]);
         px[u][1] = __builtin_amdgcn_exp2f(s[kt][qt][2 * h + 1]);
+      } else if (SM == SM_SCALED) {
+        px[u][0] = __builtin_amdgcn_exp2f(s[kt][qt][2 * h] * c);
+        px[u][1] = __builtin_amdgcn_exp2f(s[kt][qt][2 * h + 1] * c);
       } else {
         px[u][0] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][qt][2 * h], c, -mref[qt]));
         px[u][1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][qt][2 * h + 1], c, -mref[qt]));
@@ -787,13 +797,14 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
                p.diag[(size_t)blockIdx.x * DIAG_SLOTS + i] += dg[i];)
 }
 
-template <class MAP, int HP, int NW, bool FAST>
+template <class MAP, int HP, int NW, int SM>
 __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
   uint32_t* redo = reinterpret_cast<uint32_t*>(smem + RING_BYTES);
+  constexpr bool FAST = SM != SM_EXACT;
   if (FAST) {
     if (threadIdx.x < REDO_WORDS) redo[threadIdx.x] = 0;  // visible after the first tile barrier
-    run_pass<MAP, HP, NW, true, false>(p, smem, redo);
+    run_pass<MAP, HP, NW, SM, false>(p, smem, redo);
     // Every wavefront has left the first pass: its marks are in, nobody reads the ring any more and
     // the loader's last (unused) requests have landed before new ones reuse their slots.
     __builtin_amdgcn_s_waitcnt(0);
@@ -801,7 +812,7 @@ __global__ __launch_bounds__(NW * 64) void intra_fwd_kernel(const KParams p) {
     const uint32_t mine = redo[threadIdx.x & (REDO_WORDS - 1)];
     if (__builtin_amdgcn_ballot_w64(mine != 0) == 0) return;  // the usual case
   }
-  run_pass<MAP, HP, NW, false, FAST>(p, smem, redo);
+  run_pass<MAP, HP, NW, SM_EXACT, FAST>(p, smem, redo);
 }
 
 }  // namespace intra

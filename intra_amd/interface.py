@@ -33,20 +33,25 @@ def _aligned(x):
     return st[-1] == 1 and st[0] % 8 == 0 and st[1] % 8 == 0 and st[2] % 8 == 0
 
 
-SOFTMAX_MODES = {"auto": 0, "exact": 1, "fast": 2}
+# INTRA_SOFTMAX_* of include/intra_hip.h ("fast" is the older name of "folded")
+SOFTMAX_MODES = {"auto": 0, "exact": 1, "folded": 2, "scaled": 3, "fast": 2}
+_SOFTMAX_NAMES = {0: "auto", 1: "exact", 2: "folded", 3: "scaled"}
 
 
 def set_softmax_mode(mode):
-    """Softmax arithmetic of the forward kernels, process-wide: "exact" scales the fp32 scores after
-    the first product like the reference (csrc/flash_attn/src/softmax.h:65-91); "fast" folds the
-    scale into the bf16 queries and recomputes, exactly, the queries whose weight sum leaves the
-    safe exponent range; "auto" (default) picks fast up to twice the default softmax_scale."""
+    """Softmax arithmetic that calls without a `softmax=` argument get, process-wide.  "exact" scales
+    the fp32 scores after the first product and keeps a running reference like the reference
+    (csrc/flash_attn/src/softmax.h:65-91); "scaled" scales them the same way but keeps no running
+    maximum and recomputes, exactly, the queries whose weight sum leaves the safe exponent range;
+    "folded" multiplies the scale into the bf16 queries instead (about 2 % faster, error grows with
+    the magnitude of q and k); "auto" (default) is scaled up to four times the default
+    softmax_scale, exact beyond.  Meant for experiments: pass `softmax=` per call otherwise."""
     if _C.intra_set_softmax_mode(SOFTMAX_MODES[mode]) != _lib.INTRA_OK:
         raise RuntimeError(f"intra_hip: {_lib.last_error()}")
 
 
 def get_softmax_mode():
-    return {v: k for k, v in SOFTMAX_MODES.items()}[_C.intra_get_softmax_mode()]
+    return _SOFTMAX_NAMES[_C.intra_get_softmax_mode()]
 
 
 _BF16 = torch.bfloat16
@@ -112,7 +117,8 @@ def _launch(fn, fn_lse, q, k, v, pattern_id, arg0, arg1, scale, return_lse=False
     return (out, lse) if return_lse else out
 
 
-def _launch_ex(q, k, v, pattern_id, group_num, window, block, offset, n_sink, scale, return_lse):
+def _launch_ex(q, k, v, pattern_id, group_num, window, block, offset, n_sink, scale, return_lse, softmax=None):
+    flags = 0 if softmax is None else SOFTMAX_MODES[softmax]
     out = torch.empty_like(q)
     if not _aligned(out):
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
@@ -124,14 +130,32 @@ def _launch_ex(q, k, v, pattern_id, group_num, window, block, offset, n_sink, sc
                                  _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
                                  pattern_id, group_num, window, block, offset, n_sink, float(scale), stream,
                                  lse.data_ptr() if return_lse else None,
-                                 _lib.strides3(lse) if return_lse else None)
+                                 _lib.strides3(lse) if return_lse else None, flags)
+    if rc != _lib.INTRA_OK:
+        raise RuntimeError(f"intra_hip: {_lib.last_error()}")
+    return (out, lse) if return_lse else out
+
+
+def _launch_image_ex(q, k, v, pattern_id, width, text_len, scale, return_lse, softmax):
+    out = torch.empty_like(q)
+    if not _aligned(out):
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    B, S, H, _ = q.shape
+    lse = torch.empty(B, H, S, dtype=torch.float32, device=q.device) if return_lse else None
+    guard, stream = _stream_on(q.device)
+    with guard:
+        rc = _C.intra_image_fwd_ex(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, k.shape[2],
+                                   _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                                   pattern_id, width, text_len, float(scale), stream,
+                                   lse.data_ptr() if return_lse else None,
+                                   _lib.strides3(lse) if return_lse else None, SOFTMAX_MODES[softmax])
     if rc != _lib.INTRA_OK:
         raise RuntimeError(f"intra_hip: {_lib.last_error()}")
     return (out, lse) if return_lse else out
 
 
 def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_scale=None, return_lse=False,
-                   block=256, offset=0, n_sink=0):
+                   block=256, offset=0, n_sink=0, softmax=None):
     """Causal prefill attention for language models.
 
     pattern="scatter": token i attends to earlier tokens j with j % group_num == i % group_num.
@@ -144,6 +168,8 @@ def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_
     Not in the reference's signature:
     return_lse=True also returns the (batch, heads, seqlen) fp32 log-sum-exp of the scaled scores
     of every query, as `(out, lse)`.
+    softmax="exact" | "scaled" | "folded" names the kernel's softmax arithmetic for this call (see
+    set_softmax_mode); None takes the process default.
     pattern="block_scatter": tokens form blocks of `block` (a multiple of 64), block b in group
         b % group_num; a query block qb reads the earlier blocks of group (qb + offset) % group_num
         and itself where it is in that group or offset != 0, plus the first n_sink tokens.
@@ -155,9 +181,10 @@ def intra_llm_attn(q, k, v, pattern="scatter", group_num=8, window=576, softmax_
     q, k, v = _check(q, k, v)
     if pattern == "gather1" and (group_num != 8 or q.shape[1] % (group_num * group_num)):
         raise ValueError(f"gather1 needs group_num=8 and seqlen % 64 == 0, got G={group_num}, S={q.shape[1]}")
-    if pattern in EXTRA_LLM_PATTERNS:
-        return _launch_ex(q, k, v, EXTRA_LLM_PATTERNS[pattern], int(group_num), int(window), int(block),
-                          int(offset), int(n_sink), _scale(q, softmax_scale), return_lse)
+    if pattern in EXTRA_LLM_PATTERNS or softmax is not None:
+        ids = EXTRA_LLM_PATTERNS if pattern in EXTRA_LLM_PATTERNS else LLM_PATTERNS
+        return _launch_ex(q, k, v, ids[pattern], int(group_num), int(window), int(block),
+                          int(offset), int(n_sink), _scale(q, softmax_scale), return_lse, softmax)
     return _launch(_C.intra_llm_fwd, _C.intra_llm_fwd_lse, q, k, v, LLM_PATTERNS[pattern], int(group_num),
                    int(window), _scale(q, softmax_scale), return_lse)
 
@@ -261,7 +288,7 @@ def intra_image_attn_func(q, k, v, pattern="scatter", width=64, softmax_scale=No
     return _ImageAttnFunction.apply(q, k, v, pattern, width, softmax_scale)
 
 
-def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None, return_lse=False):
+def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None, return_lse=False, softmax=None):
     """Bidirectional attention for FLUX-style sequences: 512 text tokens followed by a
     width x width grid of image tokens.
 
@@ -270,12 +297,15 @@ def intra_image_attn(q, k, v, pattern="scatter", width=64, softmax_scale=None, r
     pattern="gather0": each 8 x 8 image patch attends to a 16 x 16 window around it plus all text.
 
     Width 64 (1024 x 1024 FLUX images) and 128 (2048 x 2048), as in the reference
-    (intra_attn/interface.py:59-63).  return_lse as for intra_llm_attn.
+    (intra_attn/interface.py:59-63).  return_lse and softmax as for intra_llm_attn.
     """
     q, k, v = _check(q, k, v)
     if width not in (64, 128):
         raise ValueError("image kernels are compiled for width 64 and 128")
     if q.shape[1] != TEXT_LEN + width * width:
         raise ValueError(f"expected {TEXT_LEN} text + {width}x{width} image tokens, got {q.shape[1]}")
+    if softmax is not None:
+        return _launch_image_ex(q, k, v, IMAGE_PATTERNS[pattern], int(width), TEXT_LEN, _scale(q, softmax_scale),
+                                return_lse, softmax)
     return _launch(_C.intra_image_fwd, _C.intra_image_fwd_lse, q, k, v, IMAGE_PATTERNS[pattern], int(width),
                    TEXT_LEN, _scale(q, softmax_scale), return_lse)

@@ -8,12 +8,13 @@ S x S score matrix never exists for all heads at once.  Works on CPU and GPU ten
 import torch
 
 
-def masked_attention_rows(q, k, v, mask_rows, rows=None, softmax_scale=None, chunk=1024):
+def masked_attention_rows(q, k, v, mask_rows, rows=None, softmax_scale=None, chunk=1024, out_dtype=None):
     """Attention output for a subset of query positions.
 
     q: (B, S, H, D); k, v: (B, S, Hkv, D), H % Hkv == 0; query head h uses kv head h // (H/Hkv).
     mask_rows: (len(rows), S) bool, row r belongs to query position rows[r] (all positions in
-    order if rows is None).  Returns (B, len(rows), H, D) in q.dtype.
+    order if rows is None).  Returns (B, len(rows), H, D) in q.dtype like the reference's
+    masked_attention, or in `out_dtype` (torch.float32: the result before that final rounding).
     """
     B, S, H, D = q.shape
     Hkv = k.shape[2]
@@ -24,7 +25,8 @@ def masked_attention_rows(q, k, v, mask_rows, rows=None, softmax_scale=None, chu
     rows = torch.as_tensor(rows, device=q.device, dtype=torch.long)
     kf = k.float().permute(0, 2, 3, 1)  # B, Hkv, D, S
     vf = v.float().permute(0, 2, 1, 3)  # B, Hkv, S, D
-    out = torch.empty(B, rows.numel(), H, D, dtype=q.dtype, device=q.device)
+    out_dtype = q.dtype if out_dtype is None else out_dtype
+    out = torch.empty(B, rows.numel(), H, D, dtype=out_dtype, device=q.device)
     for r0 in range(0, rows.numel(), chunk):
         idx = rows[r0:r0 + chunk]
         qf = q[:, idx].float().permute(0, 2, 1, 3)  # B, H, R, D
@@ -33,7 +35,7 @@ def masked_attention_rows(q, k, v, mask_rows, rows=None, softmax_scale=None, chu
         s = s.masked_fill(~mask_rows[r0:r0 + chunk].to(q.device)[None, None, None], float("-inf"))
         p = torch.softmax(s, dim=-1)
         o = torch.matmul(p, vf[:, :, None])  # B, Hkv, rep, R, D
-        out[:, r0:r0 + chunk] = o.reshape(B, H, idx.numel(), D).permute(0, 2, 1, 3).to(q.dtype)
+        out[:, r0:r0 + chunk] = o.reshape(B, H, idx.numel(), D).permute(0, 2, 1, 3).to(out_dtype)
     return out
 
 

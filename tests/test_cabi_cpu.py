@@ -130,12 +130,16 @@ def test_version_and_softmax_mode(lib):
     assert lib.intra_version() == major * 10000 + minor * 100 + patch
     start = lib.intra_get_softmax_mode()
     try:
-        for mode in (1, 2, 0):
+        for mode in (1, 2, 3, 0):
             assert lib.intra_set_softmax_mode(mode) == 0 and lib.intra_get_softmax_mode() == mode
-        assert lib.intra_set_softmax_mode(3) == 1 and "softmax mode" in _lib.last_error()
+        assert lib.intra_set_softmax_mode(4) == 1 and "softmax mode" in _lib.last_error()
+        assert lib.intra_set_softmax_mode(-1) == 1
         assert lib.intra_get_softmax_mode() == 0
-        intra_amd.set_softmax_mode("exact")
-        assert intra_amd.get_softmax_mode() == "exact"
+        for name in ("exact", "scaled", "folded", "auto"):
+            intra_amd.set_softmax_mode(name)
+            assert intra_amd.get_softmax_mode() == name
+        intra_amd.set_softmax_mode("fast")  # the older name of folded
+        assert intra_amd.get_softmax_mode() == "folded"
     finally:
         lib.intra_set_softmax_mode(start)
 
@@ -351,3 +355,20 @@ def test_backward_key_row_maps_equal_mask_image(lib, W, T, kind, pattern):
     assert rc == 0, _lib.last_error()
     want = oracle.mask_rows(kind, S, width=W, text_len=T).numpy().astype(np.uint8)
     assert np.array_equal(count, want), np.argwhere(count != want)[:5]
+
+
+def test_flags_of_the_ex_entry_points_are_checked_before_any_launch(lib):
+    """Unknown bits in `flags` are refused during argument validation (no GPU needed); the known
+    values get past it and fail later, on the null pointers."""
+    st = (ctypes.c_int64 * 3)(128 * 4 * 128, 4 * 128, 128)
+    for flags, text in ((4, "unknown bits in flags"), (0x80000000, "unknown bits in flags")):
+        assert lib.intra_llm_fwd_ex(None, None, None, None, 1, 128, 4, 4, st, st, st, st, 0, 8, 576, 256, 0, 0,
+                                    0.1, None, None, None, flags) == _lib.INTRA_ERR_INVALID
+        assert text in _lib.last_error()
+        assert lib.intra_image_fwd_ex(None, None, None, None, 1, 512 + 256, 4, 4, st, st, st, st, 0, 16, 512,
+                                      0.1, None, None, None, flags) == _lib.INTRA_ERR_INVALID
+        assert text in _lib.last_error()
+    for flags in (0, 1, 2, 3):
+        assert lib.intra_llm_fwd_ex(None, None, None, None, 1, 128, 4, 4, st, st, st, st, 0, 8, 576, 256, 0, 0,
+                                    0.1, None, None, None, flags) == _lib.INTRA_ERR_INVALID
+        assert "non-null device pointers" in _lib.last_error()

@@ -26,7 +26,7 @@ def test_fwd_llm_like_the_reference_calls_it(mask_id, kind, kw):
     assert len(res) == 4 and res[2] is None and res[3] is None
     mask = oracle.mask_rows(kind, 2048, device=DEV, **kw)
     assert (res[0].float() - oracle.masked_attention(q, k, v, mask).float()).abs().max().item() <= 1.6e-2
-    assert (res[1] - oracle.masked_lse_rows(q, k, mask)).abs().max().item() <= 1e-2  # default scale: scale folded into bf16 Q
+    assert (res[1] - oracle.masked_lse_rows(q, k, mask)).abs().max().item() <= 5e-3  # ln(1 + 2^-8): the sum runs over bf16-rounded weights
 
 
 @pytest.mark.parametrize("mask_id,kind", [(0, "image/scatter"), (4, "image/gather0")])

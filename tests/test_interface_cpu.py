@@ -29,11 +29,11 @@ def test_signatures_match_reference():
     assert list(llm.parameters)[:7] == ["q", "k", "v", "pattern", "group_num", "window", "softmax_scale"]
     assert [p.default for p in llm.parameters.values()][3:7] == ["scatter", 8, 576, None]
     assert {n: p.default for n, p in list(llm.parameters.items())[7:]} == {
-        "return_lse": False, "block": 256, "offset": 0, "n_sink": 0}
+        "return_lse": False, "block": 256, "offset": 0, "n_sink": 0, "softmax": None}
     img = inspect.signature(intra_amd.intra_image_attn)
     assert list(img.parameters)[:6] == ["q", "k", "v", "pattern", "width", "softmax_scale"]
     assert [p.default for p in img.parameters.values()][3:6] == ["scatter", 64, None]
-    assert {n: p.default for n, p in list(img.parameters.items())[6:]} == {"return_lse": False}
+    assert {n: p.default for n, p in list(img.parameters.items())[6:]} == {"return_lse": False, "softmax": None}
 
 
 @pytest.mark.parametrize("make", [lambda: _cpu(), lambda: _cpu(dtype=torch.float16), lambda: _cpu(D=64)])

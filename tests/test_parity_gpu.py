@@ -3,39 +3,28 @@ C ABI behind it.  Case matrix of the reference's tests/test_kernel.py:33-51 plus
 shapes, ragged / tiny / strided inputs and size-independent properties at full length.
 
 Tolerance: max-abs error <= 1.6e-2 on bf16 outputs (README.md:68-69 of the reference; its own
-test uses 2e-2 and reports ~1e-3 observed)."""
+test uses 2e-2 and reports ~1e-3 observed).  Cases whose outputs reach magnitudes where one bf16
+step exceeds that bound use the derived form of parity_util.py (fp32 oracle result + half a bf16
+step for the kernel's own rounding); they say so.
+
+The file also runs as a script with an exit code, like the reference's tests/test_kernel.py:29-57:
+`python tests/test_parity_gpu.py` walks the reference's case matrix, prints one line per case and
+exits 1 if any fails."""
+import os
+import sys
+
 import pytest
 import torch
+
+if __name__ == "__main__":  # run as a script: the repository root is not on the path yet
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
 
 import intra_amd
 import oracle
 from intra_amd import intra_image_attn, intra_llm_attn
+from parity_util import ATOL, DEV, check, make_qkv
 
 pytestmark = pytest.mark.gpu
-ATOL = 1.6e-2
-DEV = "cuda"
-
-
-def make_qkv(B, S, H, Hkv, seed=0):
-    """i.i.d. N(0,1) drawn on the CPU from a fixed seed, rounded to bf16, then moved."""
-    g = torch.Generator(device="cpu").manual_seed(seed)
-    q = torch.randn(B, S, H, 128, generator=g, dtype=torch.float32).to(torch.bfloat16)
-    k = torch.randn(B, S, Hkv, 128, generator=g, dtype=torch.float32).to(torch.bfloat16)
-    v = torch.randn(B, S, Hkv, 128, generator=g, dtype=torch.float32).to(torch.bfloat16)
-    return q.to(DEV), k.to(DEV), v.to(DEV)
-
-
-def check(out, q, k, v, kind, rows=None, scale=None, rtol=0.0, **kw):
-    S = q.shape[1]
-    assert out.shape == q.shape and out.dtype == torch.bfloat16
-    assert bool(torch.isfinite(out).all())
-    mask = oracle.mask_rows(kind, S, rows=rows, device=DEV, **kw)
-    ref = oracle.masked_attention_rows(q, k, v, mask, rows, softmax_scale=scale)
-    got = out if rows is None else out[:, rows]
-    diff = (got.float() - ref.float()).abs()
-    err = diff.max().item()
-    assert bool((diff <= ATOL + rtol * ref.float().abs()).all()), f"{kind} {kw} S={S}: max|err|={err:.3e}"
-    return err
 
 
 HEADS = [(1, 32, 8), (2, 32, 32)]
@@ -230,11 +219,9 @@ def test_oracle_on_gpu_equals_oracle_on_cpu():
 
 # fp32 log-sum-exp.  The kernel sums the bf16-rounded weights (the ones PV multiplies), each off by
 # at most 2^-8 relative, so the sum is too and the logarithm by at most ln(1 + 2^-8) = 3.9e-3.
-# With the scale folded into bf16 Q (the FAST arithmetic that the default scale gets) the scores
-# themselves move by up to 2^-9 * |scale| * sum_d |q_d k_d| (rms about 1.1e-3 of the score in nats),
-# and lse follows the largest scores: 1e-2 covers N(0,1) inputs at these scales.
-LSE_ATOL_EXACT = 5e-3
-LSE_ATOL = 1e-2
+# That holds for the exact and the scaled arithmetic alike (both scale fp32 scores), whatever the
+# size of the inputs; observed maximum over this file 3.3e-3.
+LSE_ATOL = 5e-3
 
 
 @pytest.mark.parametrize("kind,fn,S,H,Hkv,kw", [
@@ -260,7 +247,7 @@ def test_lse_output(kind, fn, S, H, Hkv, kw, scale, mode):
     mask = oracle.mask_rows(kind, S, device=DEV, **kw)
     ref = oracle.masked_lse_rows(q, k, mask, softmax_scale=scale)
     err = (lse - ref).abs().max().item()
-    assert err <= (LSE_ATOL_EXACT if mode == "exact" else LSE_ATOL), f"{kind}: lse max|err|={err:.3e}"
+    assert err <= LSE_ATOL, f"{kind}: lse max|err|={err:.3e}"
 
 
 def test_lse_depends_on_q_and_k_only():
@@ -294,8 +281,8 @@ def test_llm_window_sink(S, B, H, Hkv, kw):
     with torch.no_grad():
         out, lse = intra_llm_attn(q, k, v, "window_sink", return_lse=True, **kw)
     # Rows with two or three keys keep |out| of the size of single V rows, up to 4-5 over this many
-    # samples, where one bf16 ulp (2^-7 relative) of the output exceeds the absolute tolerance.
-    check(out, q, k, v, "llm/window_sink", rtol=2.0 ** -7, **kw)
+    # samples, where one bf16 step of the output exceeds the plain bound: derived bound.
+    check(out, q, k, v, "llm/window_sink", derived=True, **kw)
     ref = oracle.masked_lse_rows(q, k, oracle.mask_rows("llm/window_sink", S, device=DEV, **kw))
     assert (lse - ref).abs().max().item() <= LSE_ATOL
 
@@ -383,10 +370,9 @@ def test_random_llm_shapes(case):
     q, k, v = make_qkv(B, S, H, Hkv, seed=S + H)
     with torch.no_grad():
         out, lse = intra_llm_attn(q, k, v, kind, softmax_scale=scale, return_lse=True, **kw)
-    check(out, q, k, v, f"llm/{kind}", scale=scale, rtol=2.0 ** -7, **kw)
+    check(out, q, k, v, f"llm/{kind}", scale=scale, derived=True, **kw)  # short rows: outputs of the size of V rows
     ref = oracle.masked_lse_rows(q, k, oracle.mask_rows(f"llm/{kind}", S, device=DEV, **kw), softmax_scale=scale)
-    # random scales up to twice the default: the score noise of the folded scale grows with the scores
-    assert bool(((lse - ref).abs() <= LSE_ATOL + 2e-3 * ref.abs()).all())
+    assert (lse - ref).abs().max().item() <= LSE_ATOL
 
 
 # (the last three: text chunks of 32 / 64 queries, where gather0 puts the chunks of two scatter groups into
@@ -412,3 +398,45 @@ def test_image_other_text_lengths_through_the_c_abi(width, text_len, H, Hkv, pat
     check(out, q, k, v, f"image/{pattern}", width=width, text_len=text_len)
     mask = oracle.mask_rows(f"image/{pattern}", S, device=DEV, width=width, text_len=text_len)
     assert (lse - oracle.masked_lse_rows(q, k, mask)).abs().max().item() <= LSE_ATOL
+
+
+# ------------------------------------------------------------------ script entry (exit code)
+def _script_cases():
+    """The reference's matrix (tests/test_kernel.py:33-51): (name, call, kind, B, S, H, Hkv, mask arguments)."""
+    for S in (1000, 2048, 3000, 4096, 8192, 16384):
+        for B, H, Hkv in ((1, 32, 8), (2, 32, 32)):
+            for G in (2, 3, 8):
+                yield (f"llm scatter G={G}", lambda q, k, v, G=G: intra_llm_attn(q, k, v, "scatter", group_num=G),
+                       "llm/scatter", B, S, H, Hkv, dict(group_num=G))
+            if S % 64 == 0:
+                yield ("llm gather1", lambda q, k, v: intra_llm_attn(q, k, v, "gather1", group_num=8),
+                       "llm/gather1", B, S, H, Hkv, dict(group_num=8))
+            for W in (576, 1000):
+                yield (f"llm window W={W}", lambda q, k, v, W=W: intra_llm_attn(q, k, v, "window", window=W),
+                       "llm/window", B, S, H, Hkv, dict(window=W))
+    for width, H in ((64, 24), (128, 8)):
+        for B in (1, 2):
+            for pattern in ("scatter", "gather0"):
+                yield (f"image {pattern} W={width}", lambda q, k, v, p=pattern, w=width: intra_image_attn(q, k, v, p, w),
+                       f"image/{pattern}", B, 512 + width * width, H, H, dict(width=width))
+
+
+def main():
+    failed = 0
+    for name, call, kind, B, S, H, Hkv, kw in _script_cases():
+        q, k, v = make_qkv(B, S, H, Hkv)
+        with torch.no_grad():
+            out = call(q, k, v)
+        try:
+            err, ok = check(out, q, k, v, kind, **kw), True
+        except AssertionError as exc:
+            err, ok = float("nan"), False
+            print(f"    {exc}")
+        failed += not ok
+        print(f"{'PASS' if ok else 'FAIL'}  {name:22s} B={B} S={S:5d} H={H}/{Hkv}  max|err|={err:.3e}", flush=True)
+    print("ALL PASSED" if failed == 0 else f"{failed} FAILED")
+    return 1 if failed else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
