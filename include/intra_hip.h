@@ -262,11 +262,13 @@ int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint
  *
  * intra_diag_set_buffer: libraries built with -DINTRA_DIAG_TIMERS (python -m intra_amd.build --diag
  * makes intra_amd/libintra_hip_diag.so) time the phases of a work item inside the forward kernel.
- * `counters` is device memory for 8 int64 values per workgroup of the largest launch to come,
+ * `counters` is device memory for 16 int64 values per workgroup of the largest launch to come,
  * zeroed by the caller; every forward launch whose grid fits ADDS per workgroup: 100 MHz wall-clock
  * ticks of [0] item set-up, [1] the first barrier, [2] the first key block, [3] the tile loop,
  * [4] look-up of the next item, its Q request, normalisation and stores; [5] work items, [6] key
- * tiles, [7] shader cycles of the tile loops.  NULL switches it off.  A production build returns
+ * tiles, [7] shader cycles of the tile loops; [8]..[15] shader cycles at the barriers in front of
+ * the Q slots, of the first key block, of tile 0 and between tiles, each as a pair {waiting for the
+ * wavefront's own requests and LDS reads, waiting for the other wavefronts}.  NULL switches it off.  A production build returns
  * INTRA_ERR_UNSUPPORTED and never touches such a buffer.
  *
  * intra_diag_mfma_ceiling: one launch of `workgroups` x 8 wavefronts that issue nothing but bf16

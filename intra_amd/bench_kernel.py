@@ -241,6 +241,8 @@ def bench_image(args):
 
 
 PHASES = ["item set-up", "first barrier", "first key block", "tile loop", "next item, Q request, normalise, store"]
+DIAG_SLOTS = 16  # values per workgroup (csrc/intra_kernel.hip.h)
+BARRIERS = ["in front of the Q slots", "in front of the first key block", "opening tile 0", "between tiles (per tile)"]
 
 
 @torch.no_grad()
@@ -248,7 +250,7 @@ def bench_phases(args):
     """Sum over a launch of the in-kernel phase timers (see include/intra_hip.h, intra_diag_set_buffer)."""
     lib = _lib.load()
     n_wg = 4096
-    buf = torch.zeros(n_wg * 8, dtype=torch.int64, device="cuda")
+    buf = torch.zeros(n_wg * DIAG_SLOTS, dtype=torch.int64, device="cuda")
     if lib.intra_diag_set_buffer(buf.data_ptr(), buf.numel()) != 0:
         raise SystemExit(f"{_lib.last_error()}; run with INTRA_HIP_LIB={_lib.DIAG_LIB_PATH}")
     intra_amd.set_softmax_mode(args.softmax)
@@ -268,7 +270,7 @@ def bench_phases(args):
         call()
     torch.cuda.synchronize()
     lib.intra_diag_set_buffer(None, 0)
-    d = buf.view(-1, 8).double().cpu()
+    d = buf.view(-1, DIAG_SLOTS).double().cpu()
     d = d[d[:, 5] > 0] / args.iters
     items, tiles = d[:, 5].mean().item(), d[:, 6].mean().item()
     res = {"pattern": args.pattern, "seqlen": S, "softmax": args.softmax, "workgroups": d.shape[0],
@@ -282,6 +284,12 @@ def bench_phases(args):
     res["us_per_workgroup"] = {"mean": round(d[:, :5].sum(1).mean().item() / 100, 1),
                                "max": round(d[:, :5].sum(1).max().item() / 100, 1)}
     res["share_outside_tile_loop"] = round(1 - d[:, 3].sum().item() / d[:, :5].sum().item(), 4)
+    # shader cycles -> us with the clock of the tile loops; [own requests and LDS reads, other wavefronts]
+    mhz = d[:, 7].mean().item() / loop_us
+    res["barrier_wait_us"] = {}
+    for i, name in enumerate(BARRIERS):
+        per = tiles if i == 3 else items
+        res["barrier_wait_us"][name] = [round(d[:, 8 + 2 * i + j].mean().item() / mhz / per, 3) for j in range(2)]
     print(json.dumps(res), flush=True)
     return [res]
 
@@ -346,7 +354,7 @@ def main():
                    choices=["scatter", "gather1", "window", "image_scatter", "image_gather0"], help="phases: which kernel")
     p.add_argument("--seqlen", type=int, default=32768, help="phases: LLM sequence length")
     p.add_argument("--width", type=int, default=64, help="phases: image grid side")
-    p.add_argument("--softmax", default="auto", choices=["auto", "exact", "fast"], help="phases: softmax arithmetic")
+    p.add_argument("--softmax", default="auto", choices=["auto", "exact", "scaled", "folded"], help="phases: softmax arithmetic")
     p.add_argument("--out", help="optional JSON output path")
     args = p.parse_args()
     args.seqlens = [int(x) for x in args.seqlens.split(",")]

@@ -28,8 +28,8 @@
 //    the previous one still computes.  The Q rows of a work item travel in the same stream, as
 //    two ring slots in front of its key tiles: they are requested three slots ahead like any
 //    tile, arrive as whole 256-byte rows, and each wavefront picks its 32 rows out of LDS with
-//    the K operand's read pattern.  The output rows of a finished item stay in registers until
-//    the next item's first requests are out and are stored behind them.  An LDS tile is 16 groups
+//    the K operand's read pattern.  The output rows of a finished item are stored right behind its
+//    tile loop, in front of the barrier that opens the next item.  An LDS tile is 16 groups
 //    of 4 rows with an XOR chunk swizzle inside the group and 32 bytes of padding between groups,
 //    so the row-per-lane K reads and the 4-row transposing V reads are both free of bank conflicts.
 //  * The softmax reference stays 0 (weights exp2(score*c), exact after normalisation because
@@ -105,9 +105,13 @@ struct KParams {
 // Phase timers of diagnostic builds (-DINTRA_DIAG_TIMERS): wavefront 0 of every workgroup adds up,
 // over its work items, the 100 MHz wall clock spent in each phase and the shader cycles of the tile
 // loop, and stores DIAG_SLOTS values at the end: [0] item set-up, [1] first barrier, [2] first key
-// block, [3] tile loop, [4] next-item look-up, Q request, normalisation and stores, [5] work items,
-// [6] tiles, [7] shader cycles of the tile loops.  Production builds compile none of it.
-constexpr int DIAG_SLOTS = 8;
+// block, [3] tile loop, [4] next-item look-up, normalisation and output stores, [5] work items,
+// [6] tiles, [7] shader cycles of the tile loops; then shader cycles spent at the barriers, split into
+// the wait for the wavefront's own requests and LDS reads and the wait for the other wavefronts:
+// [8], [9] the barrier in front of the Q slots, [10], [11] the one in front of the first key block,
+// [12], [13] the one that opens tile 0, [14], [15] all barriers between tiles.  Production builds
+// compile none of it.
+constexpr int DIAG_SLOTS = 16;
 #ifdef INTRA_DIAG_TIMERS
 #define INTRA_DIAG(...) __VA_ARGS__
 #else
@@ -176,6 +180,25 @@ __device__ __forceinline__ float lane_quad_sum(float x) {
   auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return lane_xor32_sum(__uint_as_float(r[0]) + __uint_as_float(r[1]));
 }
+
+#ifdef INTRA_DIAG_TIMERS
+// the same, adding the shader cycles of its two waits to w[0] (own requests, LDS reads) and w[1] (barrier)
+template <int PENDING>
+__device__ __forceinline__ void tile_barrier_timed(long long* w) {
+  asm volatile("" ::: "memory");
+  const long long a = __builtin_readcyclecounter();
+  __builtin_amdgcn_s_waitcnt((PENDING & 15) | ((PENDING >> 4) << 14) | (7 << 4) | (0 << 8));
+  const long long b = __builtin_readcyclecounter();
+  __builtin_amdgcn_s_barrier();
+  const long long c = __builtin_readcyclecounter();
+  w[0] += b - a;
+  w[1] += c - b;
+  asm volatile("" ::: "memory");
+}
+#define INTRA_TILE_BARRIER(PENDING, W) tile_barrier_timed<PENDING>(W)
+#else
+#define INTRA_TILE_BARRIER(PENDING, W) tile_barrier<PENDING>()
+#endif
 
 template <int V>
 using ic = std::integral_constant<int, V>;
@@ -287,7 +310,8 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   };
   Where cw;
   if (!locate(0, cw)) return;
-  INTRA_DIAG(long long dg[DIAG_SLOTS] = {0, 0, 0, 0, 0, 0, 0, 0};)
+  long long* dgw = nullptr;  // measurement builds: the barrier counters
+  INTRA_DIAG(long long dg[DIAG_SLOTS] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}; dgw = dg + 8;)
   Feed fd = feed_for(cw, -1);
   // request the next slot of the stream into a ring slot (byte offset inside the K ring and the V ring)
   auto feed_tile = [&](int slot_off) {
@@ -371,28 +395,21 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     k0 = k1; k1 = k2; k2 = k3; k3 = tk;
   };
   // Barrier in front of a slot, leaving this wavefront's requests for the slot after the next in
-  // flight (the PER_TILE most recent operations) and, where they were issued in between, the
-  // `extra` stores of the previous work item's output (0, 8 or 9; wave-uniform).  The operation
-  // counter retires in issue order, so everything older than what is left pending has landed.
-  auto slot_barrier = [&](int extra) {
-    if (extra == 0) tile_barrier<PER_TILE>();
-    else if (extra == 8) tile_barrier<PER_TILE + 8>();
-    else tile_barrier<PER_TILE + 9>();
+  // flight (PER_TILE operations) and the `extra` stores of the previous work item's output (0, 8 or
+  // 9; wave-uniform), wherever those sit among the PER_TILE + extra most recent operations.  The
+  // operation counter retires in issue order, so everything older than that has landed.
+  auto slot_barrier = [&](int extra, long long* w) {
+    (void)w;
+    if (extra == 0) INTRA_TILE_BARRIER(PER_TILE, w);
+    else if (extra == 8) INTRA_TILE_BARRIER(PER_TILE + 8, w);
+    else INTRA_TILE_BARRIER(PER_TILE + 9, w);
   };
-  // Output of the finished work item, kept in registers until the next item's first requests are
-  // out: pk[4 * qt + m] is the 16-byte chunk 4 * m + 2 * (g4 % 2) + g4 / 2 of the row of query qt,
-  // so the four lanes of a query store 64 contiguous bytes per instruction.
-  u32x4 pk[8];
-  uint16_t* orow[2] = {nullptr, nullptr};
-  float* lse_dst = nullptr;
-  float lse_val = 0.f;
-  int held = 0;  // vector-memory operations the held output will take: 0 (nothing held), 8, or 9 with a log-sum-exp
-  auto store_held = [&] {
-    if (held == 0) return;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) *reinterpret_cast<u32x4*>(orow[i >> 2] + 32 * (i & 3)) = pk[i];
-    if (held == 9) *lse_dst = lse_val;
-  };
+  // Vector-memory stores this wavefront issued for the output of the previous work item (0, 8, or 9
+  // with a log-sum-exp).  They go out right after the item's tile loop - the wavefronts leave that
+  // loop at different times (the diagonal tile gives some of them one block more), so the early ones
+  // get their stores through the memory pipeline while the late ones still compute - and may stay in
+  // flight across the first two barriers of the next item.
+  int stored = 0;
 
   for (;;) {
   INTRA_DIAG(const long long t_a = wall_clock64();)
@@ -447,12 +464,10 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
 
   // ---------------------------------------------------------------- slot -2: the Q rows arrive
   INTRA_DIAG(const long long t_b = wall_clock64();)
-  tile_barrier<PER_TILE>();  // both Q slots have landed; the held stores are not out yet
+  const int in_flight = stored;
+  slot_barrier(in_flight, dgw);  // both Q slots have landed; behind them: the first key tile's requests, then the stores
   INTRA_DIAG(const long long t_c = wall_clock64();)
   feed_tile(k3);
-  store_held();              // behind the request, so that two more barriers can leave them in flight
-  const int in_flight = held;
-  held = 0;
   {
     // this wavefront's 32 rows: slot wave / 4 (ring slot 0 or 1 of the stream as it stands), part
     // (wave / 2) % 2, rows 32 * (wave % 2) .. of the part; read with the K operand's pattern
@@ -704,7 +719,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   // The two Q slots in front of a work item's tiles are iterations of the same kind without
   // tile work: the first reads Q out of LDS, the second computes the scores of key block 0.
   // ---------------------------------------------------------------- slot -1: the first key tile has landed
-  slot_barrier(in_flight);
+  slot_barrier(in_flight, dgw + 2);
   feed_tile(k3);
   if (jq1 < 0 && jp1 >= 0) {  // scores of key block 0, ahead of the pipeline (the tile sits in slot k1)
     load_ka(ka, 0, 0);
@@ -722,13 +737,13 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   }
   rotate();
   INTRA_DIAG(const long long t_d = wall_clock64(); const long long c_d = __builtin_readcyclecounter();)
-  slot_barrier(in_flight);  // opens tile 0; the held stores went out after the request for tile 1
+  INTRA_TILE_BARRIER(PER_TILE, dgw + 4);  // opens tile 0 (tile 1 was requested behind the stores: they are done too)
   for (int i = 0;;) {
     step(2 * i, s0, s1, ic<0>{}, ic<1>{}, k3);
     step(2 * i + 1, s1, s0, ic<1>{}, ic<0>{}, 0);
     rotate();
     if (++i == ntiles) break;
-    tile_barrier<PER_TILE>();
+    INTRA_TILE_BARRIER(PER_TILE, dgw + 6);
   }
 
   INTRA_DIAG(const long long t_e = wall_clock64(); dg[7] += __builtin_readcyclecounter() - c_d;)
@@ -738,9 +753,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   if (fd.w.round == cw.round) more = false;  // (the loader only stays on an item when it is the last)
   else if (fd.prev_round != cw.round) more = locate(cw.round + 1, nw);
 
-  // ---------------------------------------------------------------- normalise; the rows are stored later
-  // (idle wavefronts run through it as well and hold nothing: the registers of the held output
-  // are then rewritten in every work item and free during the tile loop)
+  // ---------------------------------------------------------------- normalise and store
   {
   const float l_tot[2] = {lane_quad_sum(l_acc[0]), lane_quad_sum(l_acc[1])};
   if (FAST) {
@@ -755,44 +768,46 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
                             __HIP_MEMORY_SCOPE_WORKGROUP);
   }
   const float inv[2] = {l_tot[0] > 0.f ? 1.f / l_tot[0] : 0.f, l_tot[1] > 0.f ? 1.f / l_tot[1] : 0.f};
-  // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2; the lane quarters g4 = 0, 1 store the values of
-  // query tiles 0, 1, the other two (and lanes of clamped rows) repeat them
-  held = wave_active ? (p.lse != nullptr ? 9 : 8) : 0;
-  {
-    const int qt = g4 & 1;
-    lse_dst = p.lse + (batch * p.lse_bs + hq * p.lse_hs + (qt ? qpos[1] : qpos[0]) * p.lse_ts);
-    lse_val = ((qt ? mref[1] : mref[0]) + __builtin_amdgcn_logf(qt ? l_tot[1] : l_tot[0])) * 0.6931471805599453f;
-  }
-  // The four lanes of a query hold head dims 4 * g4 .. + 3 of every 16-dim tile.  For the tile pair
-  // 2m, 2m+1 a lane quarter and its neighbour (g4 ^ 1) trade 8 bytes: the even one keeps its 4 dims
-  // of tile 2m and receives the neighbour's (the next 4 dims), the odd one does the same for tile
-  // 2m+1.  Each lane then owns one whole 16-byte chunk of the row: 4m + 2 * (g4 % 2) + g4 / 2.
+  stored = wave_active ? (p.lse != nullptr ? 9 : 8) : 0;
+  if (wave_active) {
+    // The four lanes of a query hold head dims 4 * g4 .. + 3 of every 16-dim tile.  For the tile pair
+    // 2m, 2m+1 a lane quarter and its neighbour (g4 ^ 1) trade 8 bytes: the even one keeps its 4 dims
+    // of tile 2m and receives the neighbour's (the next 4 dims), the odd one does the same for tile
+    // 2m+1.  Each lane then owns one whole 16-byte chunk of the row, 4m + 2 * (g4 % 2) + g4 / 2, and
+    // the four lanes of a query store 64 contiguous bytes per instruction.
+    const int64_t ohead = batch * p.o_bs + hq * p.o_hs + (2 * (g4 & 1) + (g4 >> 1)) * 8;
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt)
+    for (int qt = 0; qt < 2; ++qt) {
+      uint16_t* orow = p.o + (ohead + qpos[qt] * p.o_rs);
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      uint32_t w[2][2];
+      for (int m = 0; m < 4; ++m) {
+        uint32_t w[2][2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int k = 0; k < 2; ++k) {
-          floatx2 f = {oacc[2 * m + t][qt][2 * k] * inv[qt], oacc[2 * m + t][qt][2 * k + 1] * inv[qt]};
-          w[t][k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
-        }
-      auto r0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
-      auto r1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
-      pk[4 * qt + m] = u32x4{r0[0], r1[0], r0[1], r1[1]};
+          for (int k = 0; k < 2; ++k) {
+            floatx2 f = {oacc[2 * m + t][qt][2 * k] * inv[qt], oacc[2 * m + t][qt][2 * k + 1] * inv[qt]};
+            w[t][k] = __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+          }
+        auto r0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
+        auto r1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
+        *reinterpret_cast<u32x4*>(orow + 32 * m) = u32x4{r0[0], r1[0], r0[1], r1[1]};
+      }
     }
-  const int64_t ohead = batch * p.o_bs + hq * p.o_hs + (2 * (g4 & 1) + (g4 >> 1)) * 8;
-  orow[0] = p.o + (ohead + qpos[0] * p.o_rs);
-  orow[1] = p.o + (ohead + qpos[1] * p.o_rs);
+    // ln sum_j exp(scale * q.k_j) = (mref + log2 l) * ln 2; the lane quarters g4 = 0, 1 store the values of
+    // query tiles 0, 1, the other two (and lanes of clamped rows) repeat them
+    if (p.lse != nullptr) {
+      const int qt = g4 & 1;
+      p.lse[batch * p.lse_bs + hq * p.lse_hs + (qt ? qpos[1] : qpos[0]) * p.lse_ts] =
+          ((qt ? mref[1] : mref[0]) + __builtin_amdgcn_logf(qt ? l_tot[1] : l_tot[0])) * 0.6931471805599453f;
+    }
+  }
   }
   INTRA_DIAG(dg[0] += t_b - t_a; dg[1] += t_c - t_b; dg[2] += t_d - t_c; dg[3] += t_e - t_d;
              dg[4] += wall_clock64() - t_e; dg[5] += 1; dg[6] += ntiles;)
   if (!more) break;
   cw = nw;
   }  // work items
-  store_held();
   INTRA_DIAG(if (p.diag != nullptr && tid == 0) for (int i = 0; i < DIAG_SLOTS; ++i)
                p.diag[(size_t)blockIdx.x * DIAG_SLOTS + i] += dg[i];)
 }
