@@ -232,54 +232,8 @@ int plan_for(const Request& r, int hp, IntraPlan* plan) {
   return INTRA_OK;
 }
 
-// Host walk of the kernel's decomposition: sets -> row blocks -> wavefronts -> key tiles ->
-// 32-key blocks, with the same block tests and per-element bound test as the device code.
-template <class MAP>
-void model_walk(const IntraGeom& ge, int hp, int nw, uint8_t* count) {
-  const int pos = nw * 32 / hp;
-  const int S = ge.S;
-  const int n_sets = MAP::num_sets(ge);
-  const int n_mblocks = (MAP::max_nq(ge) + pos - 1) / pos;
-  for (int set = 0; set < n_sets; ++set) {
-    for (int mblk = 0; mblk < n_mblocks; ++mblk) {
-      const int t0 = mblk * pos;
-      const MAP map(ge, set, t0);
-      const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
-      if (t0 >= nq) continue;
-      const int t1 = im_min(t0 + pos, nq) - 1;
-      const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);
-      const int kt_hi = im_min(map.khi(t1), nk - 1);
-      const int ntiles = (kt_hi - kt_lo + intra::BN) / intra::BN;
-      for (int pw = 0; pw < pos / 32; ++pw) {  // the wavefronts of one head
-        const int wq0 = t0 + pw * 32;
-        if (wq0 > t1) continue;
-        const int wq_last = im_min(wq0 + 31, t1);
-        const WaveBounds wb = wave_bounds(map, wq0, wq_last);
-        for (int blk = 0; blk < (intra::BN / 32) * ntiles; ++blk) {
-          const int sb_lo = kt_lo + 32 * blk;
-          if (!block_wanted(wb, kpre, sb_lo)) continue;
-          const bool unmasked = block_unmasked(wb, kpre, sb_lo);
-          for (int l = 0; l < 32; ++l) {
-            if (wq0 + l > t1) continue;  // rows the kernel computes but never stores
-            const int tq = wq0 + l;
-            const int lo = map.klo(tq), hi = im_min(map.khi(tq), nk - 1);
-            for (int e = 0; e < 32; ++e) {
-              const int key = sb_lo + e;
-              if (!unmasked && !key_visible(key, kpre, lo, hi)) continue;
-              // an unmasked block keeps every element: clamp the loaded row like the loader does
-              const int tk = im_min(key, nk - 1);
-              const int64_t qp = map.qpos(tq), kp = map.kpos(tk);
-              uint8_t& c8 = count[qp * S + kp];
-              if (c8 < 255) ++c8;
-            }
-          }
-        }
-      }
-    }
-  }
-}
 template <class MAP> struct ModelWalk {
-  static int go(const IntraGeom& ge, int hp, int nw, uint8_t* count) { model_walk<MAP>(ge, hp, nw, count); return 0; }
+  static int go(const IntraGeom& ge, int hp, int nw, uint8_t* count) { im_model_walk<MAP>(ge, hp, nw, intra::BN, count); return 0; }
 };
 
 // CUs of the current device (cached per device; -1 if it cannot be asked)

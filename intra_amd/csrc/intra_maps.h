@@ -453,3 +453,54 @@ IM_HD bool block_unmasked(const WaveBounds& wb, int kpre, int sb_lo) {
   return sb_lo + 31 <= wb.f_hi && (sb_lo + 31 < kpre || (sb_lo >= kpre && sb_lo >= wb.f_lo));
 }
 IM_HD bool key_visible(int key, int kpre, int lo, int hi) { return key <= hi && (key < kpre || key >= lo); }
+
+// Host walk of the kernel's decomposition for one index map: sets -> row blocks of nw * 32 / hp
+// in-set queries -> wavefronts -> key tiles of `tile_keys` keys -> 32-key blocks, with the same block
+// tests and per-element bound test as the device code.  Adds 1 (saturating) to
+// count[q_pos * S + k_pos] for every score the kernel computes and keeps; `count` holds S * S bytes.
+// Host only: what the library's intra_model_mask* entry points run, and what a sanitizer build of
+// this header checks for out-of-range positions and integer overflow.
+template <class MAP>
+inline void im_model_walk(const IntraGeom& ge, int hp, int nw, int tile_keys, uint8_t* count) {
+  const int pos = nw * 32 / hp;
+  const int S = ge.S;
+  const int n_sets = MAP::num_sets(ge);
+  const int n_mblocks = (MAP::max_nq(ge) + pos - 1) / pos;
+  for (int set = 0; set < n_sets; ++set) {
+    for (int mblk = 0; mblk < n_mblocks; ++mblk) {
+      const int t0 = mblk * pos;
+      const MAP map(ge, set, t0);
+      const int nq = map.nq(), nk = map.nk(), kpre = map.kpre();
+      if (t0 >= nq) continue;
+      const int t1 = im_min(t0 + pos, nq) - 1;
+      const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);
+      const int kt_hi = im_min(map.khi(t1), nk - 1);
+      const int ntiles = (kt_hi - kt_lo + tile_keys) / tile_keys;
+      for (int pw = 0; pw < pos / 32; ++pw) {  // the wavefronts of one head
+        const int wq0 = t0 + pw * 32;
+        if (wq0 > t1) continue;
+        const int wq_last = im_min(wq0 + 31, t1);
+        const WaveBounds wb = wave_bounds(map, wq0, wq_last);
+        for (int blk = 0; blk < (tile_keys / 32) * ntiles; ++blk) {
+          const int sb_lo = kt_lo + 32 * blk;
+          if (!block_wanted(wb, kpre, sb_lo)) continue;
+          const bool unmasked = block_unmasked(wb, kpre, sb_lo);
+          for (int l = 0; l < 32; ++l) {
+            if (wq0 + l > t1) continue;  // rows the kernel computes but never stores
+            const int tq = wq0 + l;
+            const int lo = map.klo(tq), hi = im_min(map.khi(tq), nk - 1);
+            for (int e = 0; e < 32; ++e) {
+              const int key = sb_lo + e;
+              if (!unmasked && !key_visible(key, kpre, lo, hi)) continue;
+              // an unmasked block keeps every element: clamp the loaded row like the loader does
+              const int tk = im_min(key, nk - 1);
+              const int64_t qp = map.qpos(tq), kp = map.kpos(tk);
+              uint8_t& c8 = count[qp * S + kp];
+              if (c8 < 255) ++c8;
+            }
+          }
+        }
+      }
+    }
+  }
+}

@@ -1,6 +1,6 @@
 """The call pattern of the reference's LLaMA / Qwen integration (experiments/llm/llama_intra.py:
 177-221, 232-270) without model weights: a small decoder stack with random projections whose
-attention goes through intra_amd.llama_attention.intra_attention_forward, forward and backward,
+attention goes through the test helper llama_caller.sparse_attention, forward and backward,
 against the same stack on masked SDPA with the oracle's masks (what the reference trains with,
 llama_intra.py:26).  Inputs reach the kernels as transposed (B, H, S, D) views of the projection
 outputs, with GQA, an explicit scaling and the "g2s4" layer schedule: Scatter layers with stripe
@@ -15,7 +15,7 @@ import torch
 import torch.nn.functional as F
 
 import oracle
-from intra_amd.llama_attention import install_intra_llama, intra_attention_forward, set_dense_debug
+from llama_caller import attach_plans, force_dense, plan_layers, sparse_attention
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -36,12 +36,12 @@ def make_model(n_layers, seed):
 
 def masked_sdpa_forward(module, query, key, value, attention_mask=None, scaling=None, dropout=0.0, **kwargs):
     """The same interface on dense-mask SDPA, masks from the oracle."""
-    cfg, S = module._intra, query.shape[2]
-    if cfg["kind"] == "S":
-        mask = oracle.mask_rows("llm/block_scatter", S, device=DEV, group_num=cfg["num_groups"], block=cfg["scatter_block"],
-                                offset=cfg["scatter_offset"], n_sink=cfg["n_sink"])
-    elif cfg["kind"] == "W":
-        mask = oracle.mask_rows("llm/window_sink", S, device=DEV, window=cfg["window"], n_sink=cfg["n_sink"])
+    plan, S = module.intra_plan, query.shape[2]
+    if plan.kind == "scatter":
+        mask = oracle.mask_rows("llm/block_scatter", S, device=DEV, group_num=plan.group_num, block=plan.block,
+                                offset=plan.offset, n_sink=plan.n_sink)
+    elif plan.kind == "window":
+        mask = oracle.mask_rows("llm/window_sink", S, device=DEV, window=plan.window, n_sink=plan.n_sink)
     else:
         mask = torch.ones(S, S, dtype=torch.bool, device=DEV).tril()
     out = F.scaled_dot_product_attention(query, key, value, attn_mask=mask, scale=scaling, enable_gqa=True)
@@ -74,14 +74,14 @@ def rel(a, b):
 def test_g2s4_stack_forward_and_backward(S):
     B = 2
     model = make_model(8, seed=1)
-    counts = install_intra_llama(model, num_groups=2, window=200, n_sink=64, scatter_blocks=(256,),
-                                 layer_pattern="SWWW", scatter_stripe=True, scatter_n_offsets=2)
-    assert counts == (2, 6, 0)
-    assert [l.self_attn._intra["scatter_offset"] for l in model.layers if l.self_attn._intra["kind"] == "S"] == [0, 1]
+    plans = plan_layers(8, "SWWW", group_num=2, window=200, n_sink=64, blocks=(256,), stripe_offsets=2)
+    attach_plans([l.self_attn for l in model.layers], plans)
+    assert [p.kind for p in plans].count("scatter") == 2 and [p.kind for p in plans].count("window") == 6
+    assert [p.offset for p in plans if p.kind == "scatter"] == [0, 1]
     g = torch.Generator(device="cpu").manual_seed(2)
     x0 = torch.randn(B, S, HIDDEN, generator=g).to(torch.bfloat16).to(DEV)
     results = []
-    for attention in (intra_attention_forward, masked_sdpa_forward):
+    for attention in (sparse_attention, masked_sdpa_forward):
         x = x0.clone().requires_grad_(True)
         for w in params(model):
             w.grad = None
@@ -97,23 +97,24 @@ def test_g2s4_stack_forward_and_backward(S):
 
 def test_inference_decode_and_dense_branches():
     model = make_model(2, seed=3)
-    install_intra_llama(model, num_groups=2, window=128, n_sink=16, scatter_blocks=(64,), layer_pattern="SD")
+    attach_plans([l.self_attn for l in model.layers],
+                 plan_layers(2, "SD", group_num=2, window=128, n_sink=16, blocks=(64,)))
     attn_s, attn_d = model.layers[0].self_attn, model.layers[1].self_attn
     g = torch.Generator(device="cpu").manual_seed(4)
     mk = lambda h, s: torch.randn(1, h, s, D, generator=g).to(torch.bfloat16).to(DEV)
     q, k, v = mk(HQ, 700), mk(HKV, 700), mk(HKV, 700)
     with torch.no_grad():
-        out, _ = intra_attention_forward(attn_s, q, k, v, scaling=0.07)          # prefill, Scatter layer
+        out, _ = sparse_attention(attn_s, q, k, v, scaling=0.07)          # prefill, Scatter layer
         ref, _ = masked_sdpa_forward(attn_s, q, k, v, scaling=0.07)
         assert (out.float() - ref.float()).abs().max().item() <= 1.6e-2
-        out, _ = intra_attention_forward(attn_d, q, k, v)                        # dense layer
+        out, _ = sparse_attention(attn_d, q, k, v)                        # dense layer
         ref = F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=D ** -0.5, enable_gqa=True).transpose(1, 2)
         assert torch.equal(out, ref.contiguous())
-        out, _ = intra_attention_forward(attn_s, q[:, :, -1:], k, v)             # decode: one query, whole cache
+        out, _ = sparse_attention(attn_s, q[:, :, -1:], k, v)             # decode: one query, whole cache
         ref = F.scaled_dot_product_attention(q[:, :, -1:], k, v, scale=D ** -0.5, enable_gqa=True).transpose(1, 2)
         assert out.shape == (1, 1, HQ, D) and torch.equal(out, ref.contiguous())
-        set_dense_debug(model, True)                                             # teacher toggle
-        out, _ = intra_attention_forward(attn_s, q, k, v)
+        force_dense([l.self_attn for l in model.layers], True)                   # teacher toggle
+        out, _ = sparse_attention(attn_s, q, k, v)
         ref = F.scaled_dot_product_attention(q, k, v, is_causal=True, scale=D ** -0.5, enable_gqa=True).transpose(1, 2)
         assert torch.equal(out, ref.contiguous())
 
@@ -121,12 +122,12 @@ def test_inference_decode_and_dense_branches():
 def test_configuration_errors():
     model = make_model(2, seed=5)
     with pytest.raises(ValueError, match="256"):
-        install_intra_llama(model, num_groups=2, scatter_blocks=(128,), layer_pattern="S", scatter_stripe=True)
-    install_intra_llama(model, num_groups=2, scatter_blocks=(100,), layer_pattern="S")
+        plan_layers(2, "S", group_num=2, window=0, blocks=(128,), stripe_offsets=2)
+    attach_plans([l.self_attn for l in model.layers], plan_layers(2, "S", group_num=2, window=0, blocks=(100,)))
     q = torch.zeros(1, HQ, 256, D, dtype=torch.bfloat16, device=DEV)
     k = torch.zeros(1, HKV, 256, D, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(ValueError, match="multiple of 64"):
-        intra_attention_forward(model.layers[0].self_attn, q, k, k)
+        sparse_attention(model.layers[0].self_attn, q, k, k)
 
 
 @pytest.mark.timeout(600)  # the first import of transformers on a fresh machine takes a while
@@ -137,17 +138,16 @@ def test_transformers_llama_model_trains_through_the_kernels():
     transformers = pytest.importorskip("transformers")
     from transformers import AttentionInterface, LlamaConfig, LlamaForCausalLM
 
-    from intra_amd import llama_attention
-    llama_attention.register("intra")
+    AttentionInterface.register("intra", sparse_attention)
     AttentionInterface.register("intra_masked_sdpa", masked_sdpa_forward)
     cfg = LlamaConfig(hidden_size=HIDDEN, num_attention_heads=HQ, num_key_value_heads=HKV, head_dim=D, num_hidden_layers=4,
                       intermediate_size=1024, vocab_size=512, max_position_embeddings=4096)
     cfg._attn_implementation = "intra"
     torch.manual_seed(0)
     model = LlamaForCausalLM(cfg).to(torch.bfloat16).to(DEV)
-    counts = llama_attention.install_intra_llama(model, num_groups=2, window=300, n_sink=64, scatter_blocks=(256,),
-                                                 layer_pattern="SW", scatter_stripe=True, scatter_n_offsets=2)
-    assert counts == (2, 2, 0)
+    plans = plan_layers(4, "SW", group_num=2, window=300, n_sink=64, blocks=(256,), stripe_offsets=2)
+    attach_plans([layer.self_attn for layer in model.model.layers], plans)
+    assert [p.kind for p in plans] == ["scatter", "window", "scatter", "window"]
     ids = torch.randint(0, 512, (2, 1536), generator=torch.Generator().manual_seed(1)).to(DEV)
     results = []
     for impl in ("intra", "intra_masked_sdpa"):
