@@ -277,8 +277,15 @@ int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint
  * shape, 16 per iteration), on
  * operands read once from `table` (131072 bytes the caller fills: constant or random bf16 bits).
  * `sink` takes workgroups * 512 floats, `clocks` per workgroup {shader cycles, 100 MHz ticks} of
- * the loop.  Work per launch: workgroups * 8 * iters * 16 * 32768 flop.  Allocates nothing. */
+ * the loop.  Work per launch: workgroups * 8 * iters * 16 * 32768 flop.  Allocates nothing.
+ *
+ * intra_diag_ablation: 0 for every library whose results are meant to be used.  Measurement builds can
+ * be compiled with -DINTRA_ABLATE=<n> (python -m intra_amd.build --ablate <n>), which removes or doubles
+ * one ingredient of the forward kernel's inner step (1: V^T operand reads, 2: K operand re-reads, 3: the
+ * barrier between tiles, 4: exponentials, packing and row sums; 5: those issued twice) so that its cost shows
+ * in the phase timers; such a library computes wrong results on purpose and reports <n> here. */
 int intra_diag_set_buffer(long long* counters, int64_t n_values);
+int intra_diag_ablation(void);
 int intra_diag_mfma_ceiling(const void* table, float* sink, long long* clocks, int workgroups,
                             int iters, int shape, void* hip_stream);
 

@@ -49,6 +49,7 @@ SYMBOLS = {
     "intra_set_softmax_mode": (ctypes.c_int, [ctypes.c_int]),
     "intra_get_softmax_mode": (ctypes.c_int, []),
     "intra_diag_set_buffer": (ctypes.c_int, [ctypes.c_void_p, ctypes.c_int64]),
+    "intra_diag_ablation": (ctypes.c_int, []),
     "intra_diag_mfma_ceiling": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_void_p]),
     "intra_plan": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.POINTER(IntraPlan)]),
     "intra_model_mask": (ctypes.c_int, [ctypes.c_int] * 7 + [ctypes.c_void_p]),

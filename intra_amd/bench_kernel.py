@@ -15,6 +15,11 @@ build of the library (python -m intra_amd.build --diag), selected through INTRA_
     INTRA_HIP_LIB=intra_amd/libintra_hip_diag.so python -m intra_amd.bench_kernel phases \
         --pattern scatter --seqlen 32768 [--softmax exact]
 
+The same mode prices the ingredients of the kernel's inner step on an ablation build
+(python -m intra_amd.build --ablate N; the row reports N as "ablation"):
+
+    INTRA_HIP_LIB=intra_amd/libintra_hip_ablate1.so python -m intra_amd.bench_kernel phases --pattern scatter
+
 `ceiling`: what the matrix cores sustain with nothing else running, per MFMA shape (16x16x32 and
 32x32x16), with constant and with random operand bits, and the clock they run at (the board is
 power-limited):
@@ -273,7 +278,8 @@ def bench_phases(args):
     d = buf.view(-1, DIAG_SLOTS).double().cpu()
     d = d[d[:, 5] > 0] / args.iters
     items, tiles = d[:, 5].mean().item(), d[:, 6].mean().item()
-    res = {"pattern": args.pattern, "seqlen": S, "softmax": args.softmax, "workgroups": d.shape[0],
+    res = {"pattern": args.pattern, "seqlen": S, "softmax": args.softmax, "ablation": lib.intra_diag_ablation(),
+           "workgroups": d.shape[0],
            "items_per_workgroup": round(items, 2), "tiles_per_item": round(tiles / items, 2), "us_per_item": {}}
     for i, name in enumerate(PHASES):
         res["us_per_item"][name] = round(d[:, i].mean().item() / 100 / items, 3)  # 100 MHz ticks

@@ -2,6 +2,8 @@
 
     python -m intra_amd.build            # intra_amd/libintra_hip.so
     python -m intra_amd.build --diag     # intra_amd/libintra_hip_diag.so, with in-kernel phase timers
+    python -m intra_amd.build --ablate N # intra_amd/libintra_hip_ablate<N>.so: the timers plus ablation N of the
+                                         # forward kernel's inner step (wrong results on purpose; see intra_hip.h)
 
 Takes the place of the reference's CUDAExtension build (setup.py:28-68).
 """
@@ -33,11 +35,15 @@ def hipcc_path():
 DIAG_LIB = os.path.join(HERE, "libintra_hip_diag.so")
 
 
-def build(verbose=False, extra_flags=(), diag=False):
+def build(verbose=False, extra_flags=(), diag=False, ablate=0):
     """Compile the library in-tree and return its path.  diag=True builds the measurement variant
-    libintra_hip_diag.so (same sources with the in-kernel phase timers compiled in) instead."""
+    libintra_hip_diag.so (same sources with the in-kernel phase timers compiled in) instead;
+    ablate=N that variant with ablation N of the forward kernel (libintra_hip_ablate<N>.so)."""
     lib = DIAG_LIB if diag else LIB
-    if diag:
+    if ablate:
+        lib = os.path.join(HERE, f"libintra_hip_ablate{int(ablate)}.so")
+        extra_flags = ("-DINTRA_DIAG_TIMERS", f"-DINTRA_ABLATE={int(ablate)}", *extra_flags)
+    elif diag:
         extra_flags = ("-DINTRA_DIAG_TIMERS", *extra_flags)
     cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, SRC, "-o", lib + ".tmp"]
     if verbose:
@@ -54,4 +60,9 @@ def build(verbose=False, extra_flags=(), diag=False):
 
 if __name__ == "__main__":
     args = sys.argv[1:]
-    print(build(verbose=True, extra_flags=[a for a in args if a != "--diag"], diag="--diag" in args))
+    n_ablate = 0
+    if "--ablate" in args:
+        at = args.index("--ablate")
+        n_ablate = int(args[at + 1])
+        del args[at:at + 2]
+    print(build(verbose=True, extra_flags=[a for a in args if a != "--diag"], diag="--diag" in args, ablate=n_ablate))

@@ -907,6 +907,8 @@ int intra_diag_set_buffer(long long* counters, int64_t n_values) {
 #endif
 }
 
+int intra_diag_ablation(void) { return INTRA_ABLATE; }
+
 int intra_diag_mfma_ceiling(const void* table, float* sink, long long* clocks, int workgroups, int iters,
                             int shape, void* hip_stream) {
   g_err[0] = 0;

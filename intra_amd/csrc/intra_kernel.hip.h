@@ -118,6 +118,22 @@ constexpr int DIAG_SLOTS = 16;
 #define INTRA_DIAG(...)
 #endif
 
+// Ablations for measurement builds: -DINTRA_ABLATE=<n> removes one ingredient of the hand-scheduled
+// step so that its share of the time can be read off the phase timers.  The results of such a build
+// are wrong by construction (the instruction mix is what is measured), so it only compiles together
+// with the timers, and intra_diag_ablation() reports the number.
+//   1: the V^T operands are not read from LDS (a Q fragment stands in)
+//   2: the K operands are not re-read in the PV slots (the first block's stay)
+//   3: no barrier between tiles
+//   4: no exponentials, packing or row sums (Q fragments stand in for the weights)
+//   5: every exponential, packing and row-sum instruction issued twice
+#ifndef INTRA_ABLATE
+#define INTRA_ABLATE 0
+#endif
+#if INTRA_ABLATE != 0 && !defined(INTRA_DIAG_TIMERS)
+#error "INTRA_ABLATE belongs to measurement builds (-DINTRA_DIAG_TIMERS): its results are wrong on purpose"
+#endif
+
 // softmax arithmetic of a pass (template argument SM)
 constexpr int SM_EXACT = 0, SM_FOLDED = 1, SM_SCALED = 2;
 
@@ -521,7 +537,6 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   float mref[2] = {0.f, 0.f};
   float l_acc[2] = {0.f, 0.f};  // this lane's share of the two queries' weight sums
   const float c = p.scale_log2;  // |softmax_scale| * log2(e)
-  const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
 
   // operand reads: base register + compile-time byte offset
   auto kread_at = [&](int base, int off) { return *reinterpret_cast<const bf16x8*>(smem + (base + off)); };
@@ -605,7 +620,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
   // B operand of PV as they stand: the lane's 8 weights of query tile qt, packed to bf16, are
   // keys 4*g4 .. +3 and 16 + 4*g4 .. +3 of the block, the numbering the V^T reads follow.  PV
   // runs query tile 0 first, so the weights of query tile 1 are only needed 8 slots later: the
-  // exponentials of the 8 bf16 pairs are spread over slots 0..20 of the 32, the packing + row sums
+  // exponentials of the 8 bf16 pairs are spread over slots 0..20 of the 32, the packing and the row sums
   // follow two slots behind, and in EXACT mode the maximum of the next block is taken in the last
   // PV slots once its MFMA chain has drained.  sched_barrier keeps the compiler from regrouping
   // the slots.
@@ -630,26 +645,49 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
         px[u][1] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][qt][2 * h + 1], c, -mref[qt]));
       }
     };
+    uint32_t hx[8];
     auto stage_c = [&](int u) {
       floatx2 f = {px[u][0], px[u][1]};
       bf16x2 h2 = __builtin_convertvector(f, bf16x2);
-      l_acc[u >> 2] = __builtin_amdgcn_fdot2_f32_bf16(h2, ones2, l_acc[u >> 2], false);  // sums what PV multiplies
+      hx[u] = __builtin_bit_cast(uint32_t, h2);
       pb[u >> 2][2 * (u & 3)] = h2[0];
       pb[u >> 2][2 * (u & 3) + 1] = h2[1];
     };
+    // The row sum takes what PV multiplies: the two rounded weights of the pair, by one dot-product
+    // instruction with (1, 1).  (Widening them back to fp32 with a shift and a mask and adding
+    // twice - four plain instructions - measured 7 % slower: in this loop every instruction issued
+    // beside the MFMAs costs its cycles.)
+    auto stage_s = [&](int u) {
+      const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
+      l_acc[u >> 2] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, hx[u]), ones2, l_acc[u >> 2], false);
+    };
     // slot (0..31, PV slots from 16) in which the exponentials of pair u are issued
     auto valu_slot = [&](int k) {
+      if (INTRA_ABLATE == 4) return;
 #pragma unroll
       for (int u = 0; u < 8; ++u) {
         const int es = u < 4 ? 4 * u : 2 * u + 6;
         if (es == k) stage_e(u);
         if (es + 2 == k) stage_c(u);
+        if (es + 2 == k) stage_s(u);
+        if (INTRA_ABLATE == 5) {  // the same instructions once more (the sums count twice, the rest is rewritten)
+          if (es == k) {
+            asm volatile("" : "+v"(px[u][0]), "+v"(px[u][1]));
+            stage_e(u);
+          }
+          if (es + 2 == k) {
+            asm volatile("" : "+v"(px[u][0]), "+v"(px[u][1]));
+            stage_c(u);
+          }
+          if (es + 2 == k) stage_s(u);
+        }
       }
     };
+    if (INTRA_ABLATE == 4) pb[0] = qf[0][0], pb[1] = qf[1][0];
 #pragma unroll
     for (int k = 0; k < 16; ++k) {  // QK^T: k-step ks, key tile kt, query tile qt
       const int ks = k >> 2, kt = (k >> 1) & 1, qt = k & 1;
-      if ((k & 1) == 0) va[k >> 1] = vread_at(vb[k >> 2], 32 * ((k >> 1) & 1) + HALF * FBLOCK32);
+      if ((k & 1) == 0) va[k >> 1] = INTRA_ABLATE == 1 ? qf[0][(k >> 1) & 3] : vread_at(vb[k >> 2], 32 * ((k >> 1) & 1) + HALF * FBLOCK32);
       n[kt][qt] = mfma(ka[2 * ks + kt], qf[qt][ks], ks == 0 ? zero4 : n[kt][qt]);
       valu_slot(k);
       __builtin_amdgcn_sched_barrier(0);
@@ -658,7 +696,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
 #pragma unroll
     for (int k = 0; k < 16; ++k) {  // PV: query tile qt, head-dim tile dt
       const int qt = k >> 3, dt = k & 7;
-      if (k >= 8) ka[k - 8] = kread_at(kb[(k - 8) >> 1], (k & 1) * 4 * FGROUP_STRIDE + HALF * FBLOCK32);
+      if (k >= 8 && INTRA_ABLATE != 2) ka[k - 8] = kread_at(kb[(k - 8) >> 1], (k & 1) * 4 * FGROUP_STRIDE + HALF * FBLOCK32);
       oacc[dt][qt] = mfma(va[dt], pb[qt], oacc[dt][qt]);
       valu_slot(16 + k);
       if (!FAST) {
@@ -743,7 +781,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     step(2 * i + 1, s1, s0, ic<1>{}, ic<0>{}, 0);
     rotate();
     if (++i == ntiles) break;
-    INTRA_TILE_BARRIER(PER_TILE, dgw + 6);
+    if (INTRA_ABLATE != 3) INTRA_TILE_BARRIER(PER_TILE, dgw + 6);
   }
 
   INTRA_DIAG(const long long t_e = wall_clock64(); dg[7] += __builtin_readcyclecounter() - c_d;)
@@ -763,7 +801,7 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
     const uint32_t lb0 = __float_as_uint(l_tot[0]), lb1 = __float_as_uint(l_tot[1]);
     const bool bad = wave_active && ((row_valid[0] && !(lb0 >= 0x0d800000u && lb0 <= 0x5d800000u)) ||
                                      (row_valid[1] && !(lb1 >= 0x0d800000u && lb1 <= 0x5d800000u)));
-    if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0)
+    if (INTRA_ABLATE == 0 && __builtin_amdgcn_ballot_w64(bad) != 0 && lane == 0)  // (an ablated pass is not run again)
       __hip_atomic_fetch_or(&redo[(cw.round >> 5) & (REDO_WORDS - 1)], 1u << (cw.round & 31), __ATOMIC_RELAXED,
                             __HIP_MEMORY_SCOPE_WORKGROUP);
   }

@@ -372,3 +372,16 @@ def test_flags_of_the_ex_entry_points_are_checked_before_any_launch(lib):
         assert lib.intra_llm_fwd_ex(None, None, None, None, 1, 128, 4, 4, st, st, st, st, 0, 8, 576, 256, 0, 0,
                                     0.1, None, None, None, flags) == _lib.INTRA_ERR_INVALID
         assert "non-null device pointers" in _lib.last_error()
+
+
+def test_production_library_carries_no_ablation(lib, tmp_path):
+    """The library tests and callers load computes every ingredient of the kernel's step; the
+    ablations of the measurement builds do not compile without the timers."""
+    import subprocess
+    from intra_amd import build
+    assert lib.intra_diag_ablation() == 0
+    assert lib.intra_diag_set_buffer(None, 0) == _lib.INTRA_ERR_UNSUPPORTED  # no timers either
+    res = subprocess.run([build.hipcc_path(), "--offload-arch=gfx950", "-std=c++17", "-fsyntax-only", "--cuda-device-only",
+                          "-DINTRA_ABLATE=1", "-x", "hip", os.path.join(ROOT, "intra_amd", "csrc", "intra_kernel.hip.h")],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, cwd=tmp_path)
+    assert res.returncode != 0 and "INTRA_ABLATE belongs to measurement builds" in res.stdout

@@ -77,31 +77,28 @@ def test_product_never_imports_the_oracle():
                 assert "import oracle" not in text and "from oracle" not in text, f"{pkg}/{name}"
 
 
-def test_llama_caller_module_configuration_on_cpu():
-    """install_intra_llama / set_dense_debug are host logic: schedule, block and stripe offsets per layer."""
-    import types
-
-    from intra_amd.llama_attention import install_intra_llama, set_dense_debug
-    model = types.SimpleNamespace(model=types.SimpleNamespace(
-        layers=[types.SimpleNamespace(self_attn=types.SimpleNamespace()) for _ in range(32)]))
-    counts = install_intra_llama(model, num_groups=2, window=575, n_sink=64, scatter_blocks=(256,),
-                                 layer_pattern="SWWWWWWW", scatter_stripe=True, scatter_n_offsets=2)
-    assert counts == (4, 28, 0)
-    cfgs = [l.self_attn._intra for l in model.model.layers]
-    assert [c["layer_idx"] for c in cfgs if c["kind"] == "S"] == [0, 8, 16, 24]
-    assert [c["scatter_offset"] for c in cfgs if c["kind"] == "S"] == [0, 1, 0, 1]
-    assert all(c["scatter_block"] == 256 for c in cfgs if c["kind"] == "S")
-    assert all(c["window"] == 575 and c["n_sink"] == 64 for c in cfgs)
-    set_dense_debug(model, True)
-    assert all(c["dense_debug"] for c in cfgs)
+def test_llama_caller_helper_plans_layers_on_cpu():
+    """The test helper's layer planning is host logic: schedule, blocks and stripe offsets per layer,
+    and which kernel call a layer makes."""
+    from llama_caller import LayerPlan, plan_layers
+    plans = plan_layers(32, "SWWWWWWW", group_num=2, window=575, n_sink=64, blocks=(256,), stripe_offsets=2)
+    scatter = [(i, p) for i, p in enumerate(plans) if p.kind == "scatter"]
+    assert [i for i, _ in scatter] == [0, 8, 16, 24]
+    assert [p.offset for _, p in scatter] == [0, 1, 0, 1] and all(p.block == 256 for _, p in scatter)
+    assert sum(p.kind == "window" for p in plans) == 28 and all(p.n_sink == 64 for p in plans if p.kind != "dense")
+    assert plans[0].kernel_call() == ("block_scatter", dict(group_num=2, block=256, offset=0, n_sink=64))
+    assert plans[1].kernel_call() == ("window_sink", dict(window=575, n_sink=64))
     # without stripes every Scatter layer has offset 0; blocks cycle over the Scatter layers
-    counts = install_intra_llama(model, num_groups=8, scatter_blocks=(64, 128), layer_pattern="sd?w")
-    assert counts == (11, 10, 11)
-    s_cfgs = [l.self_attn._intra for l in model.model.layers if l.self_attn._intra["kind"] == "S"]
-    assert [c["scatter_block"] for c in s_cfgs[:4]] == [64, 128, 64, 128]
-    assert all(c["scatter_offset"] == 0 for c in s_cfgs)
+    plans = plan_layers(32, "sdw", group_num=8, window=512, blocks=(64, 128))
+    assert [p.kind for p in plans[:4]] == ["scatter", "dense", "window", "scatter"]
+    s_plans = [p for p in plans if p.kind == "scatter"]
+    assert [p.block for p in s_plans[:4]] == [64, 128, 64, 128] and all(p.offset == 0 for p in s_plans)
+    assert LayerPlan("dense").kernel_call() is None
+    assert LayerPlan("scatter", group_num=8).kernel_call() == ("scatter", dict(group_num=8))  # token-level Scatter
     with pytest.raises(ValueError):
-        install_intra_llama(model, num_groups=2, scatter_blocks=(128,), layer_pattern="S", scatter_stripe=True)
+        plan_layers(2, "S", group_num=2, window=0, blocks=(128,), stripe_offsets=2)
+    with pytest.raises(ValueError):
+        LayerPlan("scatter", group_num=2, block=100).kernel_call()
 
 
 def test_extension_stand_in_has_the_reference_signatures():
