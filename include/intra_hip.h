@@ -282,7 +282,8 @@ int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint
  * intra_diag_ablation: 0 for every library whose results are meant to be used.  Measurement builds can
  * be compiled with -DINTRA_ABLATE=<n> (python -m intra_amd.build --ablate <n>), which removes or doubles
  * one ingredient of the forward kernel's inner step (1: V^T operand reads, 2: K operand re-reads, 3: the
- * barrier between tiles, 4: exponentials, packing and row sums; 5: those issued twice) so that its cost shows
+ * barrier between tiles, 4: exponentials, packing and row sums; 5: those issued twice; 6: the loader's
+ * rows: the same 64 for every tile, so no address arithmetic and only L2 hits) so that its cost shows
  * in the phase timers; such a library computes wrong results on purpose and reports <n> here. */
 int intra_diag_set_buffer(long long* counters, int64_t n_values);
 int intra_diag_ablation(void);

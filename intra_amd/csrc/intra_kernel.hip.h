@@ -127,6 +127,7 @@ constexpr int DIAG_SLOTS = 16;
 //   3: no barrier between tiles
 //   4: no exponentials, packing or row sums (Q fragments stand in for the weights)
 //   5: every exponential, packing and row-sum instruction issued twice
+//   6: the loader requests the same 64 rows for every tile (no address arithmetic, and every request hits the L2)
 #ifndef INTRA_ABLATE
 #define INTRA_ABLATE 0
 #endif
@@ -349,6 +350,12 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
 #pragma unroll
       for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
         const int grp = wave * GROUPS_PER_WAVE + gi;
+        if (INTRA_ABLATE == 6) {
+          const char* row = reinterpret_cast<const char*>(p.k) + ((uint32_t)(4 * grp + ld_row) * k_rs_b + ld_col);
+          dma_group(row, lds_base + slot_off + grp * FGROUP_STRIDE);
+          dma_group(row + 256, lds_base + VBASE + slot_off + grp * FGROUP_STRIDE);
+          continue;
+        }
         const int tk = im_min(fd.rg.kt_lo + fd.tile * BN + 4 * grp + ld_row, fd.nk - 1);
         const uint32_t pos = fd.map.kpos(tk);
         dma_group(fd.kbase + ((uint64_t)pos * k_rs_b + ld_col), lds_base + slot_off + grp * FGROUP_STRIDE);
