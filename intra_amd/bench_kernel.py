@@ -20,6 +20,12 @@ The same mode prices the ingredients of the kernel's inner step on an ablation b
 
     INTRA_HIP_LIB=intra_amd/libintra_hip_ablate1.so python -m intra_amd.bench_kernel phases --pattern scatter
 
+`series`: the HIP-event time of every launch of the headline kernel, in launch order, behind a pause
+without GPU work (the board's power management answers a pause of a few milliseconds with two dozen
+slow launches):
+
+    python -m intra_amd.bench_kernel series --pauses-ms 500,50,5,0 --launches 40
+
 `ceiling`: what the matrix cores sustain with nothing else running, per MFMA shape (16x16x32 and
 32x32x16), with constant and with random operand bits, and the clock they run at (the board is
 power-limited):
@@ -300,6 +306,30 @@ def bench_phases(args):
     return [res]
 
 
+@torch.no_grad()
+def bench_series(args):
+    """Per-launch times of Scatter G=8 at --seqlen behind pauses of --pauses-ms (in that order; 0 = none)."""
+    q, k, v = qkv(args.batch, args.seqlen, args.heads, args.kv_heads)
+    call = lambda: intra_llm_attn(q, k, v, "scatter", group_num=8)
+    call()
+    torch.cuda.synchronize()
+    rows = []
+    for pause in args.pauses_ms:
+        time.sleep(pause / 1e3)
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.launches)]
+        for a, b in evs:
+            a.record()
+            call()
+            b.record()
+        torch.cuda.synchronize()
+        ms = [round(a.elapsed_time(b), 4) for a, b in evs]
+        row = {"pattern": "scatter_g8", "seqlen": args.seqlen, "pause_ms": pause, "ms": ms,
+               "mean_first_20": round(sum(ms[:20]) / len(ms[:20]), 4), "mean_rest": round(sum(ms[20:]) / max(1, len(ms[20:])), 4)}
+        rows.append(row)
+        print(json.dumps(row), flush=True)
+    return rows
+
+
 def bench_ceiling(args):
     """MFMA-only launches (8 wavefronts per CU on every CU, nothing but v_mfma_f32_16x16x32_bf16, the
     kernels' instruction, or v_mfma_f32_32x32x16_bf16, the alternative shape) with constant
@@ -339,7 +369,7 @@ def bench_ceiling(args):
 
 def main():
     p = argparse.ArgumentParser()
-    p.add_argument("mode", choices=["llm", "image", "phases", "ceiling"])
+    p.add_argument("mode", choices=["llm", "image", "phases", "ceiling", "series"])
     p.add_argument("--seqlens", default="4096,8192,16384,32768,65536")
     p.add_argument("--groups", default="2,8")
     p.add_argument("--batch", type=int, default=1)
@@ -361,13 +391,17 @@ def main():
     p.add_argument("--seqlen", type=int, default=32768, help="phases: LLM sequence length")
     p.add_argument("--width", type=int, default=64, help="phases: image grid side")
     p.add_argument("--softmax", default="auto", choices=["auto", "exact", "scaled", "folded"], help="phases: softmax arithmetic")
+    p.add_argument("--pauses-ms", default="500,50,5,0", help="series: pauses in front of each run of launches")
+    p.add_argument("--launches", type=int, default=40, help="series: launches per run")
     p.add_argument("--out", help="optional JSON output path")
     args = p.parse_args()
     args.seqlens = [int(x) for x in args.seqlens.split(",")]
     args.widths = [int(x) for x in args.widths.split(",")]
     args.groups = [int(x) for x in args.groups.split(",")]
     print(f"device: {torch.cuda.get_device_name()}  torch {torch.__version__}  peak {PEAK_BF16_TFLOPS} TFLOP/s")
-    rows = {"llm": bench_llm, "image": bench_image, "phases": bench_phases, "ceiling": bench_ceiling}[args.mode](args)
+    args.pauses_ms = [float(x) for x in args.pauses_ms.split(",")]
+    rows = {"llm": bench_llm, "image": bench_image, "phases": bench_phases, "ceiling": bench_ceiling,
+            "series": bench_series}[args.mode](args)
     if args.out:
         json.dump({"device": torch.cuda.get_device_name(), "torch": torch.__version__,
                    "args": {k: v for k, v in vars(args).items() if k != "out"}, "rows": rows},

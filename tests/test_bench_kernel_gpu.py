@@ -69,6 +69,13 @@ def test_image_rows(tmp_path):
         assert r[key + "_cpu_ms"] > r[key]
 
 
+def test_series_mode(tmp_path):
+    doc, _ = run_cli(tmp_path, "series", "--seqlen", "4096", "--pauses-ms", "20,0", "--launches", "12")
+    assert [r["pause_ms"] for r in doc["rows"]] == [20.0, 0.0]
+    for r in doc["rows"]:
+        assert len(r["ms"]) == 12 and all(0 < t < 5 for t in r["ms"])
+
+
 def test_ceiling_and_phases_modes(tmp_path):
     doc, _ = run_cli(tmp_path, "ceiling")
     assert [r["mfma"] for r in doc["rows"]] == ["16x16x32", "16x16x32", "32x32x16", "32x32x16"]
@@ -81,6 +88,10 @@ def test_ceiling_and_phases_modes(tmp_path):
     (r,) = doc["rows"]
     assert r["workgroups"] == 256 and r["items_per_workgroup"] >= 1 and r["us_per_tile"] > 0
     assert 0 < r["share_outside_tile_loop"] < 1 and all(v >= 0 for v in r["us_per_item"].values())
+    assert r["ablation"] == 0 and len(r["barrier_wait_us"]) == 4
+    assert all(own >= 0 and others >= 0 for own, others in r["barrier_wait_us"].values())
+    # the waits at the barriers are part of the phases they sit in
+    assert r["barrier_wait_us"]["in front of the Q slots"][1] <= r["us_per_item"]["first barrier"] + 0.05
     # the production library refuses the timer buffer instead of ignoring it
     res = subprocess.run([sys.executable, "-m", "intra_amd.bench_kernel", "phases", "--seqlen", "1024"], cwd=ROOT,
                          env=dict(os.environ, PYTHONPATH=ROOT), capture_output=True, text=True, timeout=300)
