@@ -90,7 +90,7 @@ int intra_image_fwd_lse(const void* q, const void* k, const void* v, void* o, in
  *   INTRA_LLM_BLOCK_SCATTER: tokens form blocks of `block` (a multiple of 64); query i in block qb
  *     sees key j <= i in block kb iff kb % group_num == (qb + offset) % group_num, or j < n_sink,
  *     or (offset != 0 and kb == qb).  0 <= offset < group_num, 0 <= n_sink <= block.  With
- *     offset != 0, block must be a multiple of 256 / min(4, largest power of two in H / Hkv).
+ *     offset != 0, block must be a multiple of 128 when H / Hkv is odd (any multiple of 64 otherwise).
  *   INTRA_LLM_WINDOW_SINK: query i sees key j <= i iff i - j < window or j < n_sink
  *     (window >= 1, n_sink >= 0; group_num ignored).
  *   flags: INTRA_SOFTMAX_* (below) for this call; other bits must be 0. */
@@ -227,7 +227,8 @@ typedef struct IntraPlan {
   int n_sets;          /* sets per (batch, kv head) (main launch) */
   int n_mblocks;       /* row blocks of the largest set (main launch) */
   int work_items;      /* row blocks to process, all launches (a multiple of 8: padded per XCD) */
-  int grid;            /* upper bound of workgroups launched: min(work_items, CUs of the device) */
+  int grid;            /* upper bound of workgroups launched; a launch uses min(work_items, what the
+                          device holds at once: one workgroup of 8 wavefronts, or two of 4, per CU) */
   int lds_bytes;       /* LDS per workgroup */
   int launches;        /* kernel launches per forward call: 1 for every pattern */
   int64_t pairs_per_head; /* unmasked (query, key) pairs per query head and batch */
@@ -240,9 +241,20 @@ int intra_plan(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, 
 /* Walks the exact set / row-block / wavefront / 32-key-block decomposition the kernel uses
  * (same index maps and block classification, compiled for the host) and adds 1 to
  * count[q_pos * S + k_pos] for every score the kernel would compute and keep.  `count` is an
- * S*S byte array the caller zeroed.  heads_per_block <= 0 means 1; waves must be 8 or <= 0. */
+ * S*S byte array the caller zeroed.  heads_per_block <= 0 means 1; waves: 8 (or <= 0), or 4 where that
+ * shape exists (half-size workgroups). */
 int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int heads_per_block,
                      int waves, uint8_t* count);
+
+/* Enumerates how the forward launch of a request deals its work items (row blocks) to a grid of
+ * `grid` workgroups of `waves` wavefronts (8, or 4 where that shape exists; grid a multiple of 8 up
+ * to plan.work_items), with the kernels' own code compiled for the host: visits[item] += 1 for every
+ * item a workgroup is dealt, item = ((pair * n_mblocks + row block) * head groups + head group),
+ * pair = (set * B + batch) * Hkv + kv head.  `visits` holds n_visits >= plan.work_items bytes the
+ * caller zeroed.  Every row block that exists must come out as 1, whatever the grid.  (No
+ * counterpart in the reference: it launches one thread block per row block.) */
+int intra_model_deal(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
+                     int waves, int grid, uint8_t* visits, int64_t n_visits);
 
 /* intra_plan / intra_model_mask for the arguments of intra_llm_fwd_ex (always 8 wavefronts). */
 int intra_plan_llm_ex(int pattern, int B, int S, int H, int Hkv, int group_num, int window,

@@ -53,6 +53,7 @@ SYMBOLS = {
     "intra_diag_mfma_ceiling": (ctypes.c_int, [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_void_p]),
     "intra_plan": (ctypes.c_int, [ctypes.c_int] * 8 + [ctypes.POINTER(IntraPlan)]),
     "intra_model_mask": (ctypes.c_int, [ctypes.c_int] * 7 + [ctypes.c_void_p]),
+    "intra_model_deal": (ctypes.c_int, [ctypes.c_int] * 10 + [ctypes.c_void_p, ctypes.c_int64]),
 }
 
 _lib = None

@@ -11,7 +11,7 @@
 #include <type_traits>
 
 #include "../../include/intra_hip.h"
-#include "intra_kernel.hip.h"
+#include "intra_kernel_narrow.hip.h"
 #include "intra_bwd_kernel.hip.h"
 #include "intra_diag.hip.h"
 
@@ -127,19 +127,19 @@ int default_hp(int ratio) { return ratio % 4 == 0 ? 4 : (ratio % 2 == 0 ? 2 : 1)
 // quarter of the wavefronts busy, and the static dealing of work items wants items of about one
 // size: 2 if the estimated cost stays within 15 % of a patch item's, else 1.  A key tile with w of
 // 8 wavefronts busy is taken to cost 5/9 + w/18 of a full one (2/3 at w = 2, measured).
-int pick_text_merge(const IntraGeom& ge, int pos, int pg) {
+int pick_text_merge(const IntraGeom& ge, int pos, int pg, int nw) {
   const int chunk = ge.text_len / 8, nimg = ge.width * ge.width / 8;
   if (chunk % 32 != 0 || 2 * chunk > pos) return 1;  // (more chunks than a row block holds share nothing)
-  auto busy = [](int w) { return 5.0 / 9 + std::min(w, 8) / 18.0; };
+  auto busy = [nw](int w) { return 5.0 / 9 + std::min(w, nw) * (8 / nw) / 18.0; };
   const double patch_item = (ge.text_len + 16 * (16 + 8 * (pg - 1))) / 64.0;
   const double cost = ge.text_len / 64.0 * busy(2 * chunk / 32) + 2 * (nimg / 64.0) * busy(chunk / 32);
   return cost <= 1.15 * patch_item ? 2 : 1;
 }
 
-bool shape_for(const Request& r, int hp, Shape* ph) {  // false: no kernel shape fits
+bool shape_for(const Request& r, int hp, Shape* ph, int nw = 8) {  // false: no kernel shape fits
   ph->geom = r.geom;
   ph->hp = hp;
-  ph->nw = 8;
+  ph->nw = nw;
   switch (r.kind) {
     case KIND_LLM_SCATTER: ph->map = MAP_LLM_SCATTER; break;
     case KIND_LLM_GATHER1: ph->map = MAP_LLM_GATHER1; break;
@@ -149,15 +149,16 @@ bool shape_for(const Request& r, int hp, Shape* ph) {  // false: no kernel shape
     case KIND_LLM_BLOCK_SCATTER:
       // with a stripe offset a row block (256 / hp queries) has to stay inside one query block
       ph->map = MAP_LLM_BLOCK_SCATTER;
-      if (r.geom.off != 0 && r.geom.blk % (8 * 32 / hp) != 0) return false;
+      if (r.geom.off != 0 && r.geom.blk % (nw * 32 / hp) != 0) return false;
       break;
     default: {
       const int np = r.geom.width / 8;
-      int pg = im_max(1, (8 * 32 / hp) / 64);
+      if (nw * 32 / hp < 64) return false;  // a row block holds whole patches
+      int pg = (nw * 32 / hp) / 64;
       while (np % pg != 0) --pg;
       ph->map = MAP_IMG_GATHER0;
       ph->geom.pg = pg;
-      ph->geom.tm = pick_text_merge(r.geom, 8 * 32 / hp, pg);
+      ph->geom.tm = pick_text_merge(r.geom, nw * 32 / hp, pg, nw);
     }
   }
   geom_finish(ph->geom);
@@ -213,29 +214,6 @@ auto by_map(int map, A&&... a) {
 template <class MAP> struct DimsOf { static LaunchDims go(const Request& r, const Shape& ph) { return dims_of<MAP>(r, ph); } };
 template <class MAP> struct PairsOf { static int64_t go(const IntraGeom& ge) { return pairs_of<MAP>(ge); } };
 
-int plan_for(const Request& r, int hp, IntraPlan* plan) {
-  Shape ph;
-  if (!shape_for(r, hp, &ph))
-    return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
-  const LaunchDims d = by_map<DimsOf>(ph.map, r, ph);
-  plan->kind = r.kind;
-  plan->heads_per_block = ph.hp;
-  plan->waves = ph.nw;
-  plan->pos_per_block = d.pos;
-  plan->n_sets = d.n_sets;
-  plan->n_mblocks = d.n_mblocks;
-  plan->launches = 1;
-  plan->lds_bytes = intra::LDS_BYTES;
-  plan->work_items = d.work_items;
-  plan->grid = plan->work_items;  // upper bound; a launch uses min(its work items, 8 * (CUs / 8))
-  plan->pairs_per_head = by_map<PairsOf>(ph.map, ph.geom);
-  return INTRA_OK;
-}
-
-template <class MAP> struct ModelWalk {
-  static int go(const IntraGeom& ge, int hp, int nw, uint8_t* count) { im_model_walk<MAP>(ge, hp, nw, intra::BN, count); return 0; }
-};
-
 // CUs of the current device (cached per device; -1 if it cannot be asked)
 int cu_count() {
   static std::atomic<int> cus[64];  // 0 = not asked yet (same answer from every thread)
@@ -249,12 +227,90 @@ int cu_count() {
   return n;
 }
 
-// One persistent workgroup per CU (LDS allows no more), in multiples of the 8 XCDs.
-int launch_grid(int work_items) {
+// Wavefronts per workgroup of a forward launch.  Half-size workgroups, two per CU, pay for every key
+// tile twice as often per query (measured: 7 % on the long rows of LLM Scatter), and gain where the
+// work items are short or few:
+//  * image gather0 (short items, and the wavefronts of one use different key tiles: the two
+//    workgroups of a CU fill each other's waits): 0.0775 -> 0.0694 ms at 1024^2, 0.266 -> 0.235 at 2048^2;
+//  * launches with so few row blocks that the CU with the most work gets at least a fifth less of it
+//    when the blocks are half as large (8 kv heads at S <= 1024: 22 -> 18 us; image scatter at
+//    1024^2, whose 576 row blocks of 256 queries are 2.25 per CU).
+// The environment variable INTRA_WAVES (4 or 8) overrides the choice for measurements, where the
+// shape exists.
+int pick_waves(const Request& r, int hp) {
+  Shape narrow, wide;
+  if (!shape_for(r, hp, &narrow, intra::NARROW_WAVES)) return 8;
+  if (!shape_for(r, hp, &wide, 8)) return intra::NARROW_WAVES;  // (block scatter with an offset: smaller row blocks fit smaller blocks)
+  if (const char* e = getenv("INTRA_WAVES")) {
+    const int n = atoi(e);
+    if (n == 8 || n == intra::NARROW_WAVES) return n;
+  }
+  if (r.kind == KIND_IMG_GATHER0) return intra::NARROW_WAVES;
+  int cus = cu_count();
+  if (cus <= 0) cus = 256;  // (planning without a device)
+  const int64_t items8 = by_map<DimsOf>(wide.map, r, wide).work_items, items4 = by_map<DimsOf>(narrow.map, r, narrow).work_items;
+  if (items8 <= 0 || items4 <= 0) return 8;
+  const int64_t share8 = 2 * ((items8 + cus - 1) / cus), share4 = (items4 + cus - 1) / cus;  // in half-size items
+  return 5 * share4 <= 4 * share8 ? intra::NARROW_WAVES : 8;
+}
+
+int plan_for(const Request& r, int hp, IntraPlan* plan) {
+  Shape ph;
+  if (!shape_for(r, hp, &ph, pick_waves(r, hp)))
+    return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
+  const LaunchDims d = by_map<DimsOf>(ph.map, r, ph);
+  plan->kind = r.kind;
+  plan->heads_per_block = ph.hp;
+  plan->waves = ph.nw;
+  plan->pos_per_block = d.pos;
+  plan->n_sets = d.n_sets;
+  plan->n_mblocks = d.n_mblocks;
+  plan->launches = 1;
+  plan->lds_bytes = ph.nw == intra::NARROW_WAVES ? intra::NARROW_LDS_BYTES : intra::LDS_BYTES;
+  plan->work_items = d.work_items;
+  plan->grid = plan->work_items;  // upper bound; a launch uses min(its work items, 8 * (CUs / 8))
+  plan->pairs_per_head = by_map<PairsOf>(ph.map, ph.geom);
+  return INTRA_OK;
+}
+
+template <class MAP> struct ModelWalk {
+  static int go(const IntraGeom& ge, int hp, int nw, uint8_t* count) { im_model_walk<MAP>(ge, hp, nw, intra::BN, count); return 0; }
+};
+
+// Host enumeration of the dealing: every workgroup of a grid asks locate_item for its items, round
+// after round, like the kernels do.
+template <class MAP, int POS>
+void deal_walk(const intra::KParams& p, int grid, int n_mblocks, uint8_t* visits) {
+  const int cols = grid / 8;
+  for (int wg = 0; wg < grid; ++wg) {
+    intra::Where w;
+    for (int round = 0; intra::locate_item<MAP, POS, false>(p, wg & 7, cols, wg >> 3, nullptr, round, w); round = w.round + 1) {
+      const int64_t pair = ((int64_t)w.set * p.B + w.batch) * p.Hkv + w.kvh;
+      uint8_t& c = visits[(pair * n_mblocks + w.mblk) * p.hgroups + w.hg];
+      if (c < 255) ++c;
+    }
+  }
+}
+template <class MAP> struct DealWalk {
+  static int go(const intra::KParams& p, int pos, int grid, int n_mblocks, uint8_t* visits) {
+    switch (pos) {
+      case 32: deal_walk<MAP, 32>(p, grid, n_mblocks, visits); break;
+      case 64: deal_walk<MAP, 64>(p, grid, n_mblocks, visits); break;
+      case 128: deal_walk<MAP, 128>(p, grid, n_mblocks, visits); break;
+      default: deal_walk<MAP, 256>(p, grid, n_mblocks, visits); break;
+    }
+    return 0;
+  }
+};
+
+// Persistent workgroups, as many as the CUs hold at once (LDS allows one of 8 wavefronts or two of
+// 4 per CU), in multiples of the 8 XCDs.
+int launch_grid(int work_items, int nw) {
   const int n = cu_count();
   if (n <= 0) return -1;
   int g = (n / 8) * 8;
   if (g < 8) g = 8;
+  g *= 8 / nw;
   return work_items < g ? work_items : g;
 }
 
@@ -275,6 +331,23 @@ int launch_sm(const intra::KParams& p, int sm, int grid, hipStream_t stream) {
   }
 }
 
+template <class MAP, int HP, int SM>
+int launch_narrow(const intra::KParams& p, int grid, hipStream_t stream) {
+  hipLaunchKernelGGL((intra::intra_fwd_kernel_narrow<MAP, HP, SM>), dim3(grid), dim3(intra::NARROW_WAVES * 64), 0, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
+  return INTRA_OK;
+}
+
+template <class MAP, int HP>
+int launch_narrow_sm(const intra::KParams& p, int sm, int grid, hipStream_t stream) {
+  switch (sm) {
+    case intra::SM_SCALED: return launch_narrow<MAP, HP, intra::SM_SCALED>(p, grid, stream);
+    case intra::SM_FOLDED: return launch_narrow<MAP, HP, intra::SM_FOLDED>(p, grid, stream);
+    default: return launch_narrow<MAP, HP, intra::SM_EXACT>(p, grid, stream);
+  }
+}
+
 template <class MAP>
 struct LaunchMap {
   static int go(const intra::KParams& p, int hp, int nw, int sm, int grid, hipStream_t stream) {
@@ -283,6 +356,12 @@ struct LaunchMap {
         case 4: return launch_sm<MAP, 4>(p, sm, grid, stream);
         case 2: return launch_sm<MAP, 2>(p, sm, grid, stream);
         case 1: return launch_sm<MAP, 1>(p, sm, grid, stream);
+      }
+    } else if (nw == intra::NARROW_WAVES) {
+      switch (hp) {
+        case 4: return launch_narrow_sm<MAP, 4>(p, sm, grid, stream);
+        case 2: return launch_narrow_sm<MAP, 2>(p, sm, grid, stream);
+        case 1: return launch_narrow_sm<MAP, 1>(p, sm, grid, stream);
       }
     }
     return fail(INTRA_ERR_UNSUPPORTED, "no kernel for heads_per_block=%d, waves=%d", hp, nw);
@@ -364,6 +443,20 @@ void set_sections(intra::KParams& p, const Request& r, const Shape& ph, const La
   p.n_slots = p.sec[0].slots + p.sec[1].slots;
 }
 
+// what locate_item needs of a launch: geometry, item counts, sections, divisors
+void set_dealing(intra::KParams& p, const Request& r, const Shape& ph, const LaunchDims& dims) {
+  p.B = r.B; p.H = r.H; p.Hkv = r.Hkv; p.ratio = r.H / r.Hkv;
+  p.geom = ph.geom;
+  p.n_sets = dims.n_sets;
+  p.n_mblocks = dims.n_mblocks;
+  p.hgroups = dims.hgroups;
+  p.n_pairs = dims.n_pairs;
+  set_sections(p, r, ph, dims);
+  p.d_nbh = make_fastdiv(r.B * r.Hkv);
+  p.d_hkv = make_fastdiv(r.Hkv);
+  p.d_hgroups = make_fastdiv(p.hgroups);
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 // `written`: the tensor is an output, so its elements may not alias (a zero stride over a dimension
@@ -434,23 +527,15 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
   p.q_rs_bytes = (uint32_t)(qs[1] * 2);
 
   Shape ph;
-  if (!shape_for(r, default_hp(H / Hkv), &ph))
-    return fail(INTRA_ERR_UNSUPPORTED, "block scatter with an offset needs block %% 256 == 0 unless H / Hkv is even (block %% 128) or a multiple of 4 (block %% 64)");
+  if (!shape_for(r, default_hp(H / Hkv), &ph, pick_waves(r, default_hp(H / Hkv))))
+    return fail(INTRA_ERR_UNSUPPORTED, "block scatter with an offset needs block %% 128 == 0 unless H / Hkv is even");
   const LaunchDims dims = by_map<DimsOf>(ph.map, r, ph);
   if (dims.work_items <= 0 || dims.n_pairs <= 0)
     return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 work items");
-  const int grid = launch_grid(dims.work_items);
+  const int grid = launch_grid(dims.work_items, ph.nw);
   if (grid <= 0)
     return fail(INTRA_ERR_HIP, "cannot query the current device: %s", hipGetErrorString(hipGetLastError()));
-  p.geom = ph.geom;
-  p.n_sets = dims.n_sets;
-  p.n_mblocks = dims.n_mblocks;
-  p.hgroups = dims.hgroups;
-  p.n_pairs = dims.n_pairs;
-  set_sections(p, r, ph, dims);
-  p.d_nbh = make_fastdiv(B * Hkv);
-  p.d_hkv = make_fastdiv(Hkv);
-  p.d_hgroups = make_fastdiv(p.hgroups);
+  set_dealing(p, r, ph, dims);
   p.diag = (int64_t)grid * intra::DIAG_SLOTS <= g_diag_values.load() ? g_diag.load() : nullptr;
   return by_map<LaunchMap>(ph.map, p, ph.hp, ph.nw, pick_softmax(scale, flags), grid, static_cast<hipStream_t>(stream));
 }
@@ -733,10 +818,10 @@ int model_mask_bwd(const Request& r, uint8_t* count) {
 
 int model_mask(const Request& r, int heads_per_block, int waves, uint8_t* count) {
   const int hp = heads_per_block > 0 ? heads_per_block : 1;
-  if ((hp != 1 && hp != 2 && hp != 4) || (waves > 0 && waves != 8))
+  if ((hp != 1 && hp != 2 && hp != 4) || (waves > 0 && waves != 8 && waves != intra::NARROW_WAVES))
     return fail(INTRA_ERR_INVALID, "no kernel for heads_per_block=%d, waves=%d", hp, waves);
   Shape ph;
-  if (!shape_for(r, hp, &ph))
+  if (!shape_for(r, hp, &ph, waves > 0 ? waves : 8))
     return fail(INTRA_ERR_UNSUPPORTED, "block size does not fit the row blocks of this head layout");
   by_map<ModelWalk>(ph.map, ph.geom, ph.hp, ph.nw, count);
   return INTRA_OK;
@@ -946,6 +1031,28 @@ int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int hea
   int rc = make_request(domain, pattern, 1, S, 1, 1, arg0, arg1, &r);
   if (rc) return rc;
   return model_mask(r, heads_per_block, waves, count);
+}
+
+int intra_model_deal(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
+                     int waves, int grid, uint8_t* visits, int64_t n_visits) {
+  g_err[0] = 0;
+  if (!visits) return fail(INTRA_ERR_INVALID, "visits pointer is null");
+  Request r;
+  int rc = make_request(domain, pattern, B, S, H, Hkv, arg0, arg1, &r);
+  if (rc) return rc;
+  if (waves != 8 && waves != intra::NARROW_WAVES) return fail(INTRA_ERR_INVALID, "waves must be 8 or 4");
+  Shape ph;
+  if (!shape_for(r, default_hp(H / Hkv), &ph, waves))
+    return fail(INTRA_ERR_UNSUPPORTED, "no kernel shape of %d wavefronts for this request", waves);
+  const LaunchDims dims = by_map<DimsOf>(ph.map, r, ph);
+  if (dims.work_items <= 0 || dims.n_pairs <= 0)
+    return fail(INTRA_ERR_UNSUPPORTED, "problem needs more than 2^31 work items");
+  if (grid < 8 || grid % 8 != 0 || grid > dims.work_items)
+    return fail(INTRA_ERR_INVALID, "grid must be a multiple of 8 in 8 .. work_items (%d)", dims.work_items);
+  if (n_visits < dims.work_items) return fail(INTRA_ERR_INVALID, "visits holds %lld values, %d needed", (long long)n_visits, dims.work_items);
+  intra::KParams p{};
+  set_dealing(p, r, ph, dims);
+  return by_map<DealWalk>(ph.map, p, dims.pos, grid, dims.n_mblocks, visits);
 }
 
 int intra_llm_fwd_ex(const void* q, const void* k, const void* v, void* o, int B, int S, int H,

@@ -217,6 +217,57 @@ __device__ __forceinline__ void tile_barrier_timed(long long* w) {
 #define INTRA_TILE_BARRIER(PENDING, W) tile_barrier<PENDING>()
 #endif
 
+// A work item: round = the workgroup's round it was dealt in
+struct Where {
+  int round, set, batch, kvh, mblk, hg;
+};
+// Key range of a row block: tiles of BN keys counted from kt_lo.
+struct Range {
+  int kt_lo, ntiles;
+};
+template <class MAP, int POS>
+IM_HD Range range_of_block(const MAP& map, int mblk) {
+  const int t0 = mblk * POS;
+  const int t1 = im_min(t0 + POS, map.nq()) - 1;
+  const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);  // first key the row block looks at
+  const int kt_hi = im_min(map.khi(t1), map.nk() - 1);
+  return Range{kt_lo, (kt_hi - kt_lo + BN) / BN};
+}
+
+// Dealing of work items.  Workgroups are handed to the 8 XCDs round-robin by id, so workgroup
+// id % 8 names the XCD.  All row blocks of one (batch, kv head, set) "pair" go to one XCD, one pair
+// after the other, longest row block first, so that the pair's K/V stays in that XCD's L2 while its
+// row blocks run.  Inside an XCD the slots are dealt to its workgroups in boustrophedon order
+// (0..w-1, w-1..0, ...), which balances the triangular causal workloads.
+// locate_item: the first non-empty work item of workgroup `wg_in_xcd` (of `wgs_per_xcd`) of XCD `xcd`
+// at or after `round`; false when there is none.  `redo` (device, second pass only): bitmap of the
+// rounds to visit.  Also runs on the host, where tests enumerate what every workgroup is dealt.
+template <class MAP, int POS, bool REDO>
+IM_HD bool locate_item(const KParams& p, int xcd, int wgs_per_xcd, int wg_in_xcd, const uint32_t* redo, int round, Where& w) {
+  for (;; ++round) {
+    const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
+    if (slot >= p.n_slots) return false;
+    if (REDO && !((redo[(round >> 5) & (REDO_WORDS - 1)] >> (round & 31)) & 1u)) continue;
+    const bool second = slot >= p.sec[0].slots;
+    const int sslot = second ? slot - p.sec[0].slots : slot;
+    const KParams::Section& sc = p.sec[second ? 1 : 0];
+    const int pq = (int)fd_div(sslot, sc.d_ipp);
+    const int pair = (sc.p_lo + pq) * 8 + xcd;
+    if (pair >= p.n_pairs) continue;
+    const int rem = sslot - pq * (int)sc.d_ipp.d;
+    const int rblk = (int)fd_div(rem, p.d_hgroups);
+    w.round = round;
+    w.set = (int)fd_div(pair, p.d_nbh);
+    const int bh = pair - w.set * (int)p.d_nbh.d;
+    w.batch = (int)fd_div(bh, p.d_hkv);
+    w.kvh = bh - w.batch * p.Hkv;
+    w.mblk = sc.mb_hi - 1 - rblk;
+    w.hg = rem - rblk * p.hgroups;
+    if (w.mblk * POS >= MAP(p.geom, w.set, w.mblk * POS).nq()) continue;
+    return true;
+  }
+}
+
 template <int V>
 using ic = std::integral_constant<int, V>;
 
@@ -238,54 +289,15 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
 
   // ---------------------------------------------------------------- persistent loop over work items
   // The grid holds about one workgroup per CU and every workgroup walks through several work items
-  // (row blocks), which saves the dispatch gap between consecutive workgroups on a CU.
-  // Workgroups are handed to the 8 XCDs round-robin by id, so workgroup id % 8 names the XCD.  All
-  // row blocks of one (batch, kv head, set) "pair" go to one XCD, one pair after the other, longest
-  // row block first, so that the pair's K/V stays in that XCD's L2 while its row blocks run.  Inside
-  // an XCD the slots are dealt to its workgroups in boustrophedon order (0..w-1, w-1..0, ...), which
-  // balances the triangular causal workloads.
+  // (row blocks), which saves the dispatch gap between consecutive workgroups on a CU; see
+  // locate_item for the order.
   const int xcd = blockIdx.x & 7;
   const int wgs_per_xcd = gridDim.x >> 3;
   const int wg_in_xcd = blockIdx.x >> 3;
-  struct Where {
-    int round, set, batch, kvh, mblk, hg;
-  };
-  // first non-empty work item of this workgroup at or after `round`
   auto locate = [&](int round, Where& w) {
-    for (;; ++round) {
-      const int slot = round * wgs_per_xcd + ((round & 1) ? wgs_per_xcd - 1 - wg_in_xcd : wg_in_xcd);
-      if (slot >= p.n_slots) return false;
-      if (REDO && !((redo[(round >> 5) & (REDO_WORDS - 1)] >> (round & 31)) & 1u)) continue;
-      const bool second = slot >= p.sec[0].slots;
-      const KParams::Section& sc = p.sec[second ? 1 : 0];
-      const int sslot = second ? slot - p.sec[0].slots : slot;
-      const int pq = (int)fd_div(sslot, sc.d_ipp);
-      const int pair = (sc.p_lo + pq) * 8 + xcd;
-      if (pair >= p.n_pairs) continue;
-      const int rem = sslot - pq * (int)sc.d_ipp.d;
-      const int rblk = (int)fd_div(rem, p.d_hgroups);
-      w.round = round;
-      w.set = (int)fd_div(pair, p.d_nbh);
-      const int bh = pair - w.set * (int)p.d_nbh.d;
-      w.batch = (int)fd_div(bh, p.d_hkv);
-      w.kvh = bh - w.batch * p.Hkv;
-      w.mblk = sc.mb_hi - 1 - rblk;
-      w.hg = rem - rblk * p.hgroups;
-      if (w.mblk * POS >= MAP(p.geom, w.set, w.mblk * POS).nq()) continue;
-      return true;
-    }
+    return locate_item<MAP, POS, REDO>(p, xcd, wgs_per_xcd, wg_in_xcd, redo, round, w);
   };
-  // Key range of a row block: tiles of BN keys counted from kt_lo.
-  struct Range {
-    int kt_lo, ntiles;
-  };
-  auto range_of = [&](const MAP& map, int mblk) {
-    const int t0 = mblk * POS;
-    const int t1 = im_min(t0 + POS, map.nq()) - 1;
-    const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);  // first key the row block looks at
-    const int kt_hi = im_min(map.khi(t1), map.nk() - 1);
-    return Range{kt_lo, (kt_hi - kt_lo + BN) / BN};
-  };
+  auto range_of = [&](const MAP& map, int mblk) { return range_of_block<MAP, POS>(map, mblk); };
 
   // ---------------------------------------------------------------- loader: HBM rows -> LDS
   // One global_load_lds_dwordx4 moves a 4-row group: lane L fetches 16 bytes of row L/16 and the
@@ -345,6 +357,16 @@ __device__ __forceinline__ void run_pass(const KParams& p, unsigned char* smem, 
           dma_group(fd.qbase + ((int64_t)(wq % HP) * p.q_hs * 2 + (uint64_t)pos * q_rs_b + ld_col),
                     lds_base + part * VBASE + slot_off + grp * FGROUP_STRIDE);
         }
+      }
+    } else if (TileRows tr; INTRA_ABLATE != 6 && map_tile_rows(fd.map, fd.rg.kt_lo + fd.tile * BN, tr)) {
+      // (wave-uniform) a tile whose key positions are affine: no per-key index arithmetic
+      const uint32_t row = (uint32_t)(ld_row * tr.row_step);
+#pragma unroll
+      for (int gi = 0; gi < GROUPS_PER_WAVE; ++gi) {
+        const int grp = wave * GROUPS_PER_WAVE + gi;
+        const uint32_t pos = (uint32_t)(tr.base + grp * tr.group_step) + row;
+        dma_group(fd.kbase + ((uint64_t)pos * k_rs_b + ld_col), lds_base + slot_off + grp * FGROUP_STRIDE);
+        dma_group(fd.vbase + ((uint64_t)pos * v_rs_b + ld_col), lds_base + VBASE + slot_off + grp * FGROUP_STRIDE);
       }
     } else {
 #pragma unroll

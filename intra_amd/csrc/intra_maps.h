@@ -206,6 +206,16 @@ struct MapImgScatter {
   IM_HD int khi(int) const { return T + nimg - 1; }
 };
 
+// Where the 64 keys of a tile sit when their positions are affine in the loader's coordinates: key
+// 4 * g + r of the tile (row r of the 4-row group g a load instruction moves) is at position
+// base + g * group_step + r * row_step.  A map that can tell (tile_rows) saves the loader the
+// per-key index arithmetic for such tiles; the others answer no (map_tile_rows below), and so does
+// any map for a tile that straddles two parts of its key list or its end.
+struct TileRows {
+  int base, group_step, row_step;
+};
+
+
 // ---- image gather0, grid queries: every 8x8 patch of grid queries sees all text plus a 16x16 grid
 // window around it (shifted inwards at the borders).  A set is a run of pg patches of one patch
 // row, so that the text keys (a prefix every query sees) and most of the window keys are shared.
@@ -248,6 +258,18 @@ struct MapImgPatch {
   }
   IM_HD int klo(int tq) const { return T + 16 * (win_start(C0 + (tq >> 6), np) - cfirst); }
   IM_HD int khi(int tq) const { return klo(tq) + 255; }
+  // A 64-key tile inside the text keys is 64 consecutive positions; one inside the window is a strip
+  // of 4 columns by 16 rows.
+  IM_HD bool tile_rows(int t_first, TileRows& a) const {
+    if (t_first + 64 <= T) {
+      a = TileRows{t_first, 4, 1};
+      return true;
+    }
+    const int u = t_first - T;
+    if (u < 0 || (u & 63) != 0 || t_first + 64 > nk()) return false;
+    a = TileRows{T + r0 * W + cfirst + 4 * (u >> 6), W, 1};
+    return true;
+  }
 };
 
 // ---- image gather0, all rows: sets 0..7 are the text-only scatter sets (the longest work items,
@@ -337,7 +359,18 @@ struct MapImgGather0F {
   IM_HD int kpos(int t) const { return is_text ? tx.kpos(t) : pa.kpos(t); }
   IM_HD int klo(int tq) const { return is_text ? tx.klo(tq) : pa.klo(tq); }
   IM_HD int khi(int tq) const { return is_text ? tx.khi(tq) : pa.khi(tq); }
+  IM_HD bool tile_rows(int t_first, TileRows& a) const { return !is_text && pa.tile_rows(t_first, a); }
 };
+
+// tile_rows of a map that has one, else false
+template <class MAP>
+IM_HD auto map_tile_rows_(const MAP& map, int t_first, TileRows& a, int) -> decltype(map.tile_rows(t_first, a)) {
+  return map.tile_rows(t_first, a);
+}
+template <class MAP>
+IM_HD bool map_tile_rows_(const MAP&, int, TileRows&, long) { return false; }
+template <class MAP>
+IM_HD bool map_tile_rows(const MAP& map, int t_first, TileRows& a) { return map_tile_rows_(map, t_first, a, 0); }
 
 // ------- LLM block scatter: blocks of blk tokens, block b in group b % G.  A query of block qb sees,
 // causally, the blocks of group (qb + off) % G, the first ns tokens ("sinks", ns <= blk) and, when

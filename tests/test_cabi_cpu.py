@@ -40,20 +40,23 @@ def test_plan_headline(lib):
 
 def test_plan_gather0_sets(lib):
     # one launch: sets of text rows (the 64 text queries of 1 or 2 scatter groups each), then sets of
-    # 4 / 2 / 1 neighbouring 8x8 patches.  At 2048 x 2048 a merged text item would be much longer than
-    # a patch item, so the chunks stay apart; at 1024 x 1024 two share a row block.
-    for H, Hkv, hp, pg in ((24, 24, 1, 4), (16, 8, 2, 2), (32, 8, 4, 1)):
+    # 2 / 1 / 1 neighbouring 8x8 patches.  At 2048 x 2048 a merged text item would be much longer than
+    # a patch item, so the chunks stay apart; so they do in the half-size row blocks at 1024 x 1024.
+    # Workgroups of 4 wavefronts where a row block then still holds a whole patch.
+    for H, Hkv, hp, waves, pg in ((24, 24, 1, 4, 2), (16, 8, 2, 4, 1), (32, 8, 4, 8, 1)):
         rc, p = _plan(lib, 1, 4, 1, 16896, H, Hkv, 128, 512)
         assert rc == 0 and p.launches == 1
-        assert (p.heads_per_block, p.waves, p.pos_per_block) == (hp, 8, 256 // hp)
+        assert (p.heads_per_block, p.waves, p.pos_per_block) == (hp, waves, waves * 32 // hp)
         assert (p.n_sets, p.n_mblocks) == (8 + 16 * 16 // pg, 1)
         assert p.work_items == 8 * -(-Hkv * p.n_sets // 8) * (H // Hkv // hp)
     rc, p = _plan(lib, 1, 4, 1, 4608, 24, 24, 64, 512)
-    assert rc == 0 and (p.n_sets, p.n_mblocks) == (4 + 8 * 8 // 4, 1)
+    assert rc == 0 and (p.n_sets, p.n_mblocks) == (8 + 8 * 8 // 2, 1)
+    # image scatter: 576 queries per set; at 1024 x 1024 the row blocks of 256 queries would be 2.25 per
+    # CU of a 256-CU device, so the launch takes half-size ones; at 2048 x 2048 it keeps the large ones
     rc, p = _plan(lib, 1, 0, 1, 4608, 24, 24, 64, 512)
-    assert rc == 0 and (p.n_sets, p.n_mblocks) == (8, 3)
+    assert rc == 0 and (p.n_sets, p.n_mblocks, p.waves) == (8, 5, 4)
     rc, p = _plan(lib, 1, 0, 1, 16896, 24, 24, 128, 512)
-    assert rc == 0 and p.launches == 1
+    assert rc == 0 and p.launches == 1 and (p.n_sets, p.n_mblocks, p.waves) == (8, 9, 8)
 
 
 @pytest.mark.parametrize("domain,pattern,kind,S,a0,a1", [
@@ -250,12 +253,15 @@ def test_ex_argument_checks(lib):
     for args, text in bad:
         assert lib.intra_plan_llm_ex(*args, ctypes.byref(p)) == _lib.INTRA_ERR_INVALID
         assert text in _lib.last_error()
-    # a stripe offset needs row blocks inside one query block: 64-token blocks with 1 q head per kv head
+    # a stripe offset needs row blocks inside one query block: with 1 q head per kv head the smallest
+    # row block has 128 queries, which 64-token blocks cannot hold
     assert lib.intra_plan_llm_ex(8, 1, 512, 4, 4, 2, 575, 64, 1, 0, ctypes.byref(p)) == _lib.INTRA_ERR_UNSUPPORTED
     assert lib.intra_plan_llm_ex(8, 1, 512, 16, 4, 2, 575, 64, 1, 0, ctypes.byref(p)) == 0
-    assert (p.heads_per_block, p.pos_per_block) == (4, 64)
+    assert (p.heads_per_block, p.pos_per_block) == (4, p.waves * 32 // 4)  # (so few row blocks: half-size workgroups)
     assert lib.intra_plan_llm_ex(8, 1, 512, 8, 4, 2, 575, 128, 1, 0, ctypes.byref(p)) == 0
-    assert (p.heads_per_block, p.pos_per_block) == (2, 128)
+    assert (p.heads_per_block, p.pos_per_block) == (2, p.waves * 32 // 2)
+    assert lib.intra_plan_llm_ex(8, 1, 512, 4, 4, 2, 575, 128, 1, 0, ctypes.byref(p)) == 0  # (only the half-size row blocks fit)
+    assert (p.heads_per_block, p.waves, p.pos_per_block) == (1, 4, 128)
     # the old patterns pass through and ignore the extra arguments
     q = _lib.IntraPlan()
     assert lib.intra_plan_llm_ex(0, 1, 32768, 32, 8, 8, 576, 0, 0, 0, ctypes.byref(p)) == 0

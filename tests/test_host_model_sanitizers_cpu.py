@@ -30,11 +30,37 @@ static IntraGeom geom(int S) {
   return ge;
 }
 
+static int g_waves = 8;  // wavefronts per workgroup of the walks
+
+// tiles whose key positions a map calls affine (tile_rows): every key where the formula puts it
+template <class MAP>
+static void check_tile_rows(const IntraGeom& ge, int pos) {
+  const int n_sets = MAP::num_sets(ge);
+  for (int set = 0; set < n_sets; ++set) {
+    const int nq = MAP(ge, set, 0).nq();
+    for (int t0 = 0; t0 < nq; t0 += pos) {
+      const MAP map(ge, set, t0);
+      const int kt_lo = MAP::kHasPrefix ? 0 : map.klo(t0);
+      for (int t_first = kt_lo; t_first < map.nk() + 64; t_first += 64) {
+        TileRows tr;
+        if (!map_tile_rows(map, t_first, tr)) continue;
+        for (int g = 0; g < 16; ++g)
+          for (int r = 0; r < 4; ++r)
+            if (t_first + 4 * g + r >= map.nk() || tr.base + g * tr.group_step + r * tr.row_step != map.kpos(t_first + 4 * g + r)) {
+              printf("tile_rows differs from kpos: set %d t0 %d tile %d key %d\n", set, t0, t_first, 4 * g + r);
+              exit(3);
+            }
+      }
+    }
+  }
+}
+
 template <class MAP>
 static long walk(IntraGeom ge, int hp) {
   geom_finish(ge);
+  check_tile_rows<MAP>(ge, g_waves * 32 / hp);
   std::vector<uint8_t> count((size_t)ge.S * ge.S, 0);  // exact size: a position >= S lands in a redzone
-  im_model_walk<MAP>(ge, hp, 8, 64, count.data());
+  im_model_walk<MAP>(ge, hp, g_waves, 64, count.data());
   long pairs = 0;
   for (uint8_t c : count) {
     if (c > 1) { printf("a score was computed %d times\n", (int)c); exit(2); }
@@ -45,7 +71,9 @@ static long walk(IntraGeom ge, int hp) {
 
 int main() {
   const int hps[] = {1, 2, 4};
+  for (int waves : {8, 4})
   for (int hp : hps) {
+    g_waves = waves;
     for (int S : {1, 5, 63, 64, 65, 257, 777, 1000, 2048}) {
       for (int G : {1, 2, 3, 8, 13}) { IntraGeom ge = geom(S); ge.G = G; printf("scatter %d %d %d %ld\n", hp, S, G, walk<MapLlmScatter>(ge, hp)); }
       for (int G : {2, 8}) { IntraGeom ge = geom(S); ge.G = G; printf("gather1 %d %d %d %ld\n", hp, S, G, walk<MapLlmGather1>(ge, hp)); }
@@ -60,20 +88,25 @@ int main() {
         printf("block_scatter %d %d %d %d %d %d %ld\n", hp, S, G, blk, off, ns, walk<MapLlmBlockScatter>(ge, hp));
       }
     }
-    for (int width : {16, 24, 40}) for (int text : {8, 72, 200}) {
+    for (int width : {16, 24, 40}) for (int text : {8, 72, 128, 200}) {
       IntraGeom ge = geom(text + width * width); ge.width = width; ge.text_len = text;
       printf("image_scatter %d %d %d %ld\n", hp, width, text, walk<MapImgScatter>(ge, hp));
-      int pg = 256 / hp / 64; if (pg < 1) pg = 1;
+      int pg = waves * 32 / hp / 64;
+      if (pg < 1) continue;  // (a row block holds whole patches)
       while ((width / 8) % pg != 0) --pg;
       for (int tm : {1, 2}) {
         const int chunk = text / 8;
-        if (tm == 2 && (chunk % 32 != 0 || 2 * chunk > 256 / hp)) continue;  // what the launcher allows
+        if (tm == 2 && (chunk % 32 != 0 || 2 * chunk > waves * 32 / hp)) continue;  // what the launcher allows
         ge.pg = pg; ge.tm = tm;
         printf("image_gather0 %d %d %d %ld\n", hp, width, text, walk<MapImgGather0F>(ge, hp));
       }
     }
   }
+  g_waves = 8;
   { IntraGeom ge = geom(512 + 32 * 32); ge.width = 32; ge.text_len = 512; ge.pg = 4; ge.tm = 2;
+    printf("image_gather0 1 32 512 %ld\n", walk<MapImgGather0F>(ge, 1)); }
+  g_waves = 4;
+  { IntraGeom ge = geom(512 + 32 * 32); ge.width = 32; ge.text_len = 512; ge.pg = 2; ge.tm = 1;
     printf("image_gather0 1 32 512 %ld\n", walk<MapImgGather0F>(ge, 1)); }
   printf("done\n");
   return 0;

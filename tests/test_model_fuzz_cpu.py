@@ -37,6 +37,19 @@ def test_scatter_and_gather1(lib, S, G, hp, gather):
 
 
 @settings(**COMMON)
+@given(S=st.integers(1, 1400), G=st.integers(1, 40), W=st.integers(64, 3000), hp=st.sampled_from([1, 2, 4]),
+       pattern=st.sampled_from([0, 1, 4]))
+def test_half_size_workgroups(lib, S, G, W, hp, pattern):
+    """The same walks with row blocks of 4 wavefronts (128 / hp queries)."""
+    count = np.zeros((S, S), dtype=np.uint8)
+    rc = lib.intra_model_mask(0, pattern, S, G, W, hp, 4, count.ctypes.data)
+    assert rc == 0, _lib.last_error()
+    kind = {0: "llm/scatter", 1: "llm/gather1", 4: "llm/window"}[pattern]
+    kw = dict(window=W) if pattern == 4 else dict(group_num=G)
+    assert torch.equal(torch.from_numpy(count), oracle.mask_rows(kind, S, **kw).to(torch.uint8))
+
+
+@settings(**COMMON)
 @given(S=st.integers(1, 1400), W=st.integers(64, 3000), hp=st.sampled_from([1, 2, 4]))
 def test_aligned_window(lib, S, W, hp):
     rc, count = _walk(lib, 4, S, hp, window=W)
@@ -67,13 +80,17 @@ def test_block_scatter(lib, S, G, blk64, off, ns_frac, hp):
     assert torch.equal(count, want.to(torch.uint8))
 
 
-@settings(max_examples=25, deadline=None, suppress_health_check=[HealthCheck.function_scoped_fixture])
-@given(w8=st.integers(2, 7), t8=st.integers(1, 40), hp=st.sampled_from([1, 2, 4]), gather0=st.booleans())
-def test_image_patterns(lib, w8, t8, hp, gather0):
+@settings(max_examples=40, deadline=None, suppress_health_check=[HealthCheck.function_scoped_fixture])
+@given(w8=st.integers(2, 7), t8=st.integers(1, 40), hp=st.sampled_from([1, 2, 4]), gather0=st.booleans(),
+       waves=st.sampled_from([8, 4]))
+def test_image_patterns(lib, w8, t8, hp, gather0, waves):
     W, T = 8 * w8, 8 * t8
     S = T + W * W
     count = np.zeros((S, S), dtype=np.uint8)
-    rc = lib.intra_model_mask(1, 4 if gather0 else 0, S, W, T, hp, 8, count.ctypes.data)
+    rc = lib.intra_model_mask(1, 4 if gather0 else 0, S, W, T, hp, waves, count.ctypes.data)
+    if gather0 and waves * 32 // hp < 64:  # a row block holds whole 8x8 patches
+        assert rc == _lib.INTRA_ERR_UNSUPPORTED
+        return
     assert rc == 0, _lib.last_error()
     kind = "image/gather0" if gather0 else "image/scatter"
     want = oracle.mask_rows(kind, S, width=W, text_len=T)
