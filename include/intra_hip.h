@@ -167,7 +167,7 @@ int intra_llm_bwd(const void* q, const void* k, const void* v, const void* o, co
                   const int64_t dk_strides[3], const int64_t dv_strides[3],
                   const int64_t lse_strides[3], int pattern, int group_num, int window, int block,
                   int offset, int n_sink, float softmax_scale, void* hip_stream);
-/* Floats of workspace that intra_llm_bwd needs for such a call (B*H*S rounded up to 4, plus with
+/* Floats of workspace that intra_llm_bwd needs for such a call (twice B*H*S rounded up to 4, plus with
  * sinks chunks * B * Hkv * min(n_sink, S) * 128, the queries being cut into chunks so that the
  * sink pass has about one workgroup per CU; the size is the same on every device - it allows for
  * 320 CUs, and a launch never splits finer than that); -1 if the request is invalid or unsupported

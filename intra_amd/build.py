@@ -22,6 +22,10 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # inputs are finite by contract; -inf is used for masking, so infinities stay honoured
     "-fno-honor-nans",
+    # MFMA results may live in ordinary registers also where a kernel needs more than 256 of them (the
+    # fused dK / dV kernel, one wavefront per SIMD): only pure accumulators then go to the other half of
+    # the register file.  Kernels below that size compile to the same code with and without it.
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 

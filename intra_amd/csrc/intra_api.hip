@@ -545,7 +545,7 @@ int run(int domain, const void* q, const void* k, const void* v, void* o, int B,
 template <class RMAP, int MODE, int HP, bool PARTIAL = false>
 int launch_bwd(const intra::BParams& p, int64_t grid, hipStream_t stream) {
   if (grid <= 0 || grid > 0x7fffffff) return fail(INTRA_ERR_UNSUPPORTED, "backward needs more than 2^31 workgroups");
-  hipLaunchKernelGGL((intra::intra_bwd_kernel<RMAP, MODE, HP, PARTIAL>), dim3((unsigned)grid), dim3(512), 0, stream, p);
+  hipLaunchKernelGGL((intra::intra_bwd_kernel<RMAP, MODE, HP, PARTIAL>), dim3((unsigned)grid), dim3(intra::bwd_waves(MODE) * 64), 0, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(INTRA_ERR_HIP, "kernel launch failed: %s", hipGetErrorString(e));
   return INTRA_OK;
@@ -576,19 +576,20 @@ int run_bwd_dq(intra::BParams p, int hp, hipStream_t stream) {
   }
 }
 
-// dK then dV over a key-row map: row blocks of 256 keys of one kv head, all query heads of its
-// group streamed past
+// One launch over a key-row map: row blocks of one kv head's keys (32 per wavefront of the mode's
+// workgroups), all query heads of its group streamed past
 template <class R, bool PARTIAL, int MODE>
 int run_bwd_keys_mode(intra::BParams p, hipStream_t stream) {
+  constexpr int rows = intra::bwd_waves(MODE) * 32;
   const int64_t pairs = (int64_t)R::num_sets(p.geom) * p.B * p.Hkv;
   p.hgroups = 1;
-  p.n_rblocks = (R::max_rows(p.geom) + 255) / 256;
+  p.n_rblocks = (R::max_rows(p.geom) + rows - 1) / rows;
   return launch_bwd<R, MODE, 1, PARTIAL>(p, bwd_grid(p, pairs), stream);
 }
+// dK and dV over a key-row map, in one pass
 template <class R>
 int run_bwd_keys(const intra::BParams& p, hipStream_t stream) {
-  if (int rc = run_bwd_keys_mode<R, false, intra::BWD_DK>(p, stream)) return rc;
-  return run_bwd_keys_mode<R, false, intra::BWD_DV>(p, stream);
+  return run_bwd_keys_mode<R, false, intra::BWD_DKV>(p, stream);
 }
 
 // Queries per workgroup of the pass over the `ns` leading keys (LLM sinks, image text keys): about
@@ -635,10 +636,11 @@ int leading_keys(const Request& r) {
   return 0;
 }
 
-// floats of workspace: D = rowsum(dO o O) per (batch, head, token), then the partial sums of the leading keys
+// floats of workspace: -D = -rowsum(dO o O) and lse * log2(e) per (batch, head, token), then the partial
+// sums of the leading keys
 int64_t bwd_dsum_floats(int B, int S, int H) { return ((int64_t)B * H * S + 3) & ~(int64_t)3; }
 int64_t bwd_workspace_floats(const Request& r, int cus) {
-  int64_t n = bwd_dsum_floats(r.B, r.S, r.H);
+  int64_t n = 2 * bwd_dsum_floats(r.B, r.S, r.H);
   const int ns = leading_keys(r);
   if (ns > 0) {
     const int chunk = leading_chunk(r.S, r.B, r.Hkv, ns, cus);
@@ -693,7 +695,8 @@ int run_bwd(int domain, const void* q, const void* k, const void* v, const void*
   p.dout = static_cast<const uint16_t*>(dout);
   p.lse = lse;
   p.dsum = dsum;
-  p.part = dsum + bwd_dsum_floats(B, S, H);
+  p.l2 = dsum + bwd_dsum_floats(B, S, H);
+  p.part = p.l2 + bwd_dsum_floats(B, S, H);
   p.dq = static_cast<uint16_t*>(dq);
   p.dk = static_cast<uint16_t*>(dk);
   p.dv = static_cast<uint16_t*>(dv);
@@ -780,12 +783,12 @@ float* noalloc_scratch() {
 // Host walk of the backward decomposition: count[q * S + k] += 1 for every (query, key) pair that
 // the dK / dV launches (key-row maps with their `store` rule, then the sink pass) multiply.
 template <class R>
-void bwd_walk(const IntraGeom& ge, uint8_t* count) {
+void bwd_walk(const IntraGeom& ge, uint8_t* count, int rows) {  // rows: keys per row block of the launch
   const int S = ge.S;
   for (int set = 0; set < R::num_sets(ge); ++set)
-    for (int r0 = 0; r0 < R::max_rows(ge); r0 += 256) {
+    for (int r0 = 0; r0 < R::max_rows(ge); r0 += rows) {
       const R m(ge, set, r0);
-      const int r1 = std::min(r0 + 256, m.n_rows()) - 1;
+      const int r1 = std::min(r0 + rows, m.n_rows()) - 1;
       for (int t = r0; t <= r1; ++t) {
         const int kp = m.row_pos(t);
         if (!m.store(kp)) continue;
@@ -802,16 +805,16 @@ int model_mask_bwd(const Request& r, uint8_t* count) {
   Shape sh;
   if (!shape_for(r, 1, &sh)) return fail(INTRA_ERR_UNSUPPORTED, "no kernel shape for this request");
   switch (sh.map) {
-    case MAP_LLM_SCATTER: bwd_walk<intra::KeyRowsOf<MapLlmScatter>>(sh.geom, count); break;
-    case MAP_LLM_GATHER1: bwd_walk<intra::KeyRowsOf<MapLlmGather1>>(sh.geom, count); break;
-    case MAP_LLM_WINDOW: bwd_walk<intra::KeyRowsOf<MapLlmWindow>>(sh.geom, count); break;
-    case MAP_LLM_BLOCK_SCATTER: bwd_walk<intra::KeyRowsBlockScatter>(sh.geom, count); break;
-    case MAP_LLM_WINDOW_SINK: bwd_walk<intra::KeyRowsWindowSink>(sh.geom, count); break;
+    case MAP_LLM_SCATTER: bwd_walk<intra::KeyRowsOf<MapLlmScatter>>(sh.geom, count, intra::bwd_waves(intra::BWD_DKV) * 32); break;
+    case MAP_LLM_GATHER1: bwd_walk<intra::KeyRowsOf<MapLlmGather1>>(sh.geom, count, intra::bwd_waves(intra::BWD_DKV) * 32); break;
+    case MAP_LLM_WINDOW: bwd_walk<intra::KeyRowsOf<MapLlmWindow>>(sh.geom, count, intra::bwd_waves(intra::BWD_DKV) * 32); break;
+    case MAP_LLM_BLOCK_SCATTER: bwd_walk<intra::KeyRowsBlockScatter>(sh.geom, count, intra::bwd_waves(intra::BWD_DKV) * 32); break;
+    case MAP_LLM_WINDOW_SINK: bwd_walk<intra::KeyRowsWindowSink>(sh.geom, count, intra::bwd_waves(intra::BWD_DKV) * 32); break;
     default: return fail(INTRA_ERR_UNSUPPORTED, "backward: no kernels for this pattern");
   }
   if (leading_keys(r) > 0) {
     sh.geom.sink_chunk = leading_chunk(r.S, 1, 1, leading_keys(r), MODEL_CUS);
-    bwd_walk<intra::KeyRowsSinks>(sh.geom, count);
+    bwd_walk<intra::KeyRowsSinks>(sh.geom, count, 256);
   }
   return INTRA_OK;
 }
@@ -834,12 +837,12 @@ int model_mask_image_bwd(const Request& r, uint8_t* count) {
   ge.ns = ge.text_len;  // the text keys are the leading keys every query sees
   ge.sink_chunk = leading_chunk(r.S, 1, 1, ge.ns, MODEL_CUS);
   if (r.kind == KIND_IMG_SCATTER) {
-    bwd_walk<intra::KeyRowsImgGroup<false>>(ge, count);
+    bwd_walk<intra::KeyRowsImgGroup<false>>(ge, count, intra::bwd_waves(intra::BWD_DKV) * 32);
   } else {
-    bwd_walk<intra::KeyRowsImgWindow>(ge, count);
-    bwd_walk<intra::KeyRowsImgGroup<true>>(ge, count);
+    bwd_walk<intra::KeyRowsImgWindow>(ge, count, intra::bwd_waves(intra::BWD_DKV) * 32);
+    bwd_walk<intra::KeyRowsImgGroup<true>>(ge, count, intra::bwd_waves(intra::BWD_DKV) * 32);
   }
-  bwd_walk<intra::KeyRowsText>(ge, count);
+  bwd_walk<intra::KeyRowsText>(ge, count, 256);
   return INTRA_OK;
 }
 

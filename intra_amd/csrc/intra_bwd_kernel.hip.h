@@ -22,12 +22,27 @@
 
 namespace intra {
 
-enum BwdMode : int { BWD_DQ = 0, BWD_DK = 1, BWD_DV = 2 };
+// BWD_DKV forms dK and dV in one pass (the scores of a block are computed once for both): the two
+// accumulators, the K and V fragments of the key rows, the scores, dP, both sets of weights and the
+// operand ring need more than the 256 registers of a wavefront at two wavefronts per SIMD, so this
+// mode runs workgroups of 4 wavefronts, one per SIMD, with up to 512 registers each.
+// f(ic<B>{}), f(ic<B + 1>{}), ..., f(ic<E - 1>{})
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(ic<B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
+enum BwdMode : int { BWD_DQ = 0, BWD_DK = 1, BWD_DV = 2, BWD_DKV = 3 };
+constexpr int bwd_waves(int mode) { return mode == BWD_DKV ? 4 : 8; }
 
 struct BParams {
   const uint16_t *q, *k, *v, *o, *dout;  // bf16 (B, S, heads, 128)
   const float* lse;                      // (B, H, S): ln sum exp(scale * q.k) from the forward pass
-  float* dsum;                           // (B, H, S) workspace: D = rowsum(dO o O), written by dQ, read by dK
+  float* dsum;                           // (B, H, S) workspace: -D = -rowsum(dO o O), written by dQ, read by dK
+  float* l2;                             // (B, H, S) workspace: lse * log2(e), written by dQ, read by dK / dV
   uint16_t *dq, *dk, *dv;
   float* part;  // partial sums of the sink pass: (chunk, batch, kv head, sink, 128) fp32
   // element strides: batch, row (token), head
@@ -46,6 +61,13 @@ struct BParams {
 
 constexpr int BWD_SLOT = 2 * FTILE + 512;  // two tiles and 2 x 64 column scalars
 constexpr int BWD_LDS_BYTES = 3 * BWD_SLOT;
+constexpr int bwd_ring_slots(int mode) { return mode == BWD_DKV ? 4 : 3; }
+
+// 64 lanes x 4 bytes from per-lane global addresses to 256 consecutive LDS bytes at lds_addr (the
+// active lanes' parts of them), like dma_group
+__device__ __forceinline__ void dma_dwords(const void* gsrc, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dword %0, off" : : "v"(gsrc), "s"(lds_addr) : "memory");
+}
 
 // RMAP: row map (intra_bwd_maps.h).  PARTIAL: the results are partial sums over the set's columns,
 // written as fp32 to p.part instead of bf16 to dk / dv (sink pass).
@@ -56,12 +78,19 @@ constexpr int BWD_LDS_BYTES = 3 * BWD_SLOT;
 // operand of the accumulation, whose 32-column reduction is numbered slot s of lane quarter g4 =
 // column 16*(s/4) + 4*g4 + s%4; the transposing reads of the X tile follow that numbering.
 template <class RMAP, int MODE, int HP, bool PARTIAL = false>
-__global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
-  constexpr int NW = 8;
+__global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const BParams p) {
+  constexpr int NW = bwd_waves(MODE);
+  constexpr bool HAS_DP = MODE != BWD_DV;                    // forms dP and dS
+  constexpr bool HAS_V = MODE == BWD_DV || MODE == BWD_DKV;  // accumulates dV (weights P)
+  static_assert(!(MODE == BWD_DKV && PARTIAL), "the partial sums of the sink pass come from the separate modes");
   constexpr bool ROWS_ARE_QUERIES = MODE == BWD_DQ;
   constexpr int POS = ROWS_ARE_QUERIES ? NW * 32 / HP : NW * 32;  // rows per row block (of one head)
 
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[BWD_LDS_BYTES];
+  // BWD_DKV: a step of its single wavefront per SIMD is about as long as a tile takes to arrive, so
+  // its ring is one slot deeper and a tile has two steps to land; the column scalars travel the same
+  // way (every wavefront requests those of 16 columns) instead of through registers.
+  constexpr bool DEEP = MODE == BWD_DKV;
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[bwd_ring_slots(MODE) * BWD_SLOT];
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
   const int tid = threadIdx.x;
@@ -148,6 +177,7 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   // [rt][ks]: lane holds row 16 * rt + l16, head dims 32 * ks + 8 * g4 .. +7
   bf16x8 r1f[2][4], r2f[2][4];
   float L2_row[2] = {0.f, 0.f}, D_row[2] = {0.f, 0.f};
+  auto load_rows = [&] {
 #pragma unroll
   for (int rt = 0; rt < 2; ++rt) {
     const uint16_t *a1, *a2;
@@ -161,7 +191,7 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
       r1f[rt][ks] = *reinterpret_cast<const bf16x8*>(a1 + ks * 32);
-      if (MODE != BWD_DV) r2f[rt][ks] = *reinterpret_cast<const bf16x8*>(a2 + ks * 32);
+      if (HAS_DP) r2f[rt][ks] = *reinterpret_cast<const bf16x8*>(a2 + ks * 32);
     }
     if (ROWS_ARE_QUERIES) {
       // D = dO . O of the row: this lane's 32 head dims, then the rest from the other three lanes of the row
@@ -175,9 +205,14 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
       }
       D_row[rt] = lane_quad_sum(part);
       L2_row[rt] = p.lse[batch * p.lse_bs + hq * p.lse_hs + rpos[rt] * p.lse_ts] * 1.4426950408889634f;
-      if (row_valid[rt] && g4 == 0) p.dsum[batch * p.ds_bs + hq * p.ds_hs + rpos[rt]] = D_row[rt];
+      if (row_valid[rt] && g4 == 0) {  // what the dK / dV launches need per query, in the form they use it
+        p.dsum[batch * p.ds_bs + hq * p.ds_hs + rpos[rt]] = -D_row[rt];
+        p.l2[batch * p.ds_bs + hq * p.ds_hs + rpos[rt]] = L2_row[rt];
+      }
     }
   }
+  };
+  if (!DEEP) load_rows();  // (the deep ring requests its first tiles before them, see below)
 
   // ---------------------------------------------------------------- LDS addressing (as in the forward kernel)
   const int ld_row = lane >> 4;
@@ -207,14 +242,39 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
         (__attribute__((address_space(3))) bf16x4*)(smem + o2 + 4 * FGROUP_STRIDE));
     return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
   };
+  // Deep ring: the same reads from per-lane bases that carry the ring slot (b0: the step's slot, b1:
+  // the next one's), advanced once per step, so that everything else is a compile-time offset
+  int kb0[4], kb1[4], vb0[4], sb0 = 0, sb1 = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    kb0[i] = kaddr[i];
+    kb1[i] = BWD_SLOT + kaddr[i];
+    vb0[i] = vaddr[i];
+  }
+  sb0 = 2 * FTILE + 16 * g4;
+  sb1 = BWD_SLOT + 2 * FTILE + 16 * g4;
+  auto kread_b = [&](const int (&kb)[4], int off, int f) {
+    return *reinterpret_cast<const bf16x8*>(smem + (kb[f >> 1] + (off + (f & 1) * 4 * FGROUP_STRIDE)));
+  };
+  auto vread_b = [&](int off, int dt) {
+    const int o2 = vb0[dt >> 1] + (off + 32 * (dt & 1));
+    bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(smem + o2));
+    bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+        (__attribute__((address_space(3))) bf16x4*)(smem + (o2 + 4 * FGROUP_STRIDE)));
+    return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
   auto mfma = [](bf16x8 a, bf16x8 b, floatx4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); };
   const floatx4 zero4 = {0.f, 0.f, 0.f, 0.f};
 
   floatx4 acc[8][2];  // [head-dim tile][row tile]: head dims 16 * dt + 4 * g4 .. + 3 of row 16 * rt + l16
+  floatx4 acc_v[MODE == BWD_DKV ? 8 : 1][2];  // BWD_DKV: dV (acc is dK)
 #pragma unroll
   for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) acc[dt][rt] = zero4;
+    for (int rt = 0; rt < 2; ++rt) {
+      acc[dt][rt] = zero4;
+      if (MODE == BWD_DKV) acc_v[dt][rt] = zero4;
+    }
   const float c2 = p.scale_log2;
   const float s_hidden = c2 >= 0.f ? -INFINITY : INFINITY;  // score that gives exp2(s * c2 - lse) = 0
 
@@ -254,30 +314,47 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
     c2hs = p.do_hs * 2;
   }
   auto col_pos = [&](int c) { return map.col_pos(c); };
+  // dK / dV take a tile once per query head of the group, head after head: the rows' positions are
+  // worked out for the first head and kept for the others
+  uint32_t pos_kept[16 / NW] = {};
+  int64_t spos_kept = 0;
+  auto load_group = [&](const Cursor& cu, int slot_off, int gi) {  // this wavefront's group gi of both tiles
+    const int grp = wave * (16 / NW) + gi;
+    if (ROWS_ARE_QUERIES || cu.head == 0) pos_kept[gi] = col_pos(im_min(cb + cu.tile * BN + 4 * grp + ld_row, n_cols - 1));
+    const uint32_t pos = pos_kept[gi];
+    dma_group(c1base + (cu.head * c1hs + (uint64_t)pos * c1rs + ld_col), lds_base + slot_off + grp * FGROUP_STRIDE);
+    dma_group(c2base + (cu.head * c2hs + (uint64_t)pos * c2rs + ld_col),
+              lds_base + slot_off + FTILE + grp * FGROUP_STRIDE);
+  };
   auto load_tile = [&](const Cursor& cu, int slot_off) {
 #pragma unroll
-    for (int gi = 0; gi < 2; ++gi) {
-      const int grp = wave * 2 + gi;
-      const int c = im_min(cb + cu.tile * BN + 4 * grp + ld_row, n_cols - 1);
-      const uint32_t pos = col_pos(c);
-      dma_group(c1base + (cu.head * c1hs + (uint64_t)pos * c1rs + ld_col), lds_base + slot_off + grp * FGROUP_STRIDE);
-      dma_group(c2base + (cu.head * c2hs + (uint64_t)pos * c2rs + ld_col),
-                lds_base + slot_off + FTILE + grp * FGROUP_STRIDE);
+    for (int gi = 0; gi < 16 / NW; ++gi) load_group(cu, slot_off, gi);
+  };
+  // requests per wavefront for one step of the deep ring: its groups of both tiles and two for the scalars
+  constexpr int DEEP_REQUESTS = 2 * (16 / NW) + 2;
+  auto load_scalars = [&](const Cursor& cu, int slot_off) {  // (deep ring) lse * log2(e) and -D of the step's 64 columns
+    static_assert(!DEEP || NW == 4, "16 columns per wavefront");
+    if (cu.head == 0) spos_kept = col_pos(im_min(cb + cu.tile * BN + lane, n_cols - 1));
+    if ((lane >> 4) == wave) {
+      const int64_t pos = spos_kept;
+      const int hcol = kvh * p.ratio + cu.head;
+      dma_dwords(p.l2 + (batch * p.ds_bs + hcol * p.ds_hs + pos), lds_base + slot_off + 2 * FTILE);
+      dma_dwords(p.dsum + (batch * p.ds_bs + hcol * p.ds_hs + pos), lds_base + slot_off + 2 * FTILE + 256);
     }
   };
-  // column scalars of a step (dK / dV): wavefront 0 fetches lse * log2(e) and D of its 64 columns
+  // column scalars of a step (dK / dV): wavefront 0 fetches lse * log2(e) and -D of its 64 columns
   float sc_l = 0.f, sc_d = 0.f;
   auto fetch_scalars = [&](const Cursor& cu) {
-    if (!ROWS_ARE_QUERIES && wave == 0) {
+    if (!ROWS_ARE_QUERIES && !DEEP && wave == 0) {
       const int c = im_min(cb + cu.tile * BN + lane, n_cols - 1);
       const int64_t pos = col_pos(c);
       const int hcol = kvh * p.ratio + cu.head;
-      sc_l = p.lse[batch * p.lse_bs + hcol * p.lse_hs + pos * p.lse_ts] * 1.4426950408889634f;
-      if (MODE == BWD_DK) sc_d = p.dsum[batch * p.ds_bs + hcol * p.ds_hs + pos];
+      sc_l = p.l2[batch * p.ds_bs + hcol * p.ds_hs + pos];
+      if (HAS_DP) sc_d = p.dsum[batch * p.ds_bs + hcol * p.ds_hs + pos];
     }
   };
   auto put_scalars = [&](int slot_off) {
-    if (!ROWS_ARE_QUERIES && wave == 0) {
+    if (!ROWS_ARE_QUERIES && !DEEP && wave == 0) {
       float* sc = reinterpret_cast<float*>(smem + slot_off + 2 * FTILE);
       sc[lane] = sc_l;
       sc[64 + lane] = sc_d;
@@ -299,29 +376,53 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   // of its first block are formed at the end of step t) and the tile of step t+2 is in flight.
   Cursor cur{ROWS_ARE_QUERIES ? 0 : ntiles - 1, 0};  // step being computed
   Cursor ld = cur;                                   // step being requested
-  for (int t = 0; t < 2 && t < n_steps; ++t) {
+  // (Deep ring: one slot more, the tile of step t+3 is requested during step t, and the barrier of a
+  // step leaves the most recent request in flight where one was made during the step before.)
+  for (int t = 0; t < (DEEP ? 3 : 2) && t < n_steps; ++t) {
     load_tile(ld, t * BWD_SLOT);
+    if (DEEP) load_scalars(ld, t * BWD_SLOT);
     fetch_scalars(ld);
     put_scalars(t * BWD_SLOT);
     advance(ld);
   }
-  int slot0 = 0, slot1 = BWD_SLOT, slot2 = 2 * BWD_SLOT;
+  // The deep ring's barriers leave requests in flight.  The row operands are ordinary loads the
+  // compiler waits for at their first use, inside the main loop, with a count that knows nothing of
+  // the requests issued by hand - it would wait for those as well, every time round.  So they are
+  // requested here, behind the first tiles (whose latency they share), and land here, once.
+  if (DEEP) {
+    load_rows();
+    __builtin_amdgcn_s_waitcnt((0 & 15) | (7 << 4) | (15 << 8) | (0 << 14));  // vmcnt(0)
+  }
+  int slot0 = 0, slot1 = BWD_SLOT, slot2 = 2 * BWD_SLOT, slot3 = 3 * BWD_SLOT;
+  bool fresh = DEEP && n_steps >= 3;  // the most recent request is for the step after the next
   floatx4 s_cur[2][2];  // [ct][rt]
 #pragma unroll
   for (int t = 0; t < 4; ++t) s_cur[t >> 1][t & 1] = zero4;
   bool have = false;  // s_cur and fr hold what a previous block prepared for the one that comes next
   // One slot is one MFMA; an LDS operand serves two consecutive slots (the two row tiles).
-  constexpr int NFRAG = MODE == BWD_DV ? 16 : 24;  // LDS operands per block
-  constexpr int LA = MODE == BWD_DK ? 4 : MODE == BWD_DV ? 8 : 6;  // operands between the request of one and its use
+  constexpr int NFRAG = MODE == BWD_DV ? 16 : MODE == BWD_DKV ? 32 : 24;  // LDS operands per block
+  constexpr int LA = MODE == BWD_DK ? 4 : MODE == BWD_DQ ? 6 : 8;  // operands between the request of one and its use
   static_assert(NFRAG % LA == 0, "a block must leave the ring where the next block expects it");
-  constexpr int WS = MODE == BWD_DV ? 4 : 16;      // slot of the first weight stage
-  constexpr int WSTEP = MODE == BWD_DV ? 1 : 2;    // slots from one stage to the next
+  // slot of the first weight stage and slots from one stage to the next; BWD_DKV: of the dS stages
+  // (its P stages run in slots 5 .. 15, in front of the dV accumulation)
+  constexpr int WS = MODE == BWD_DV ? 4 : MODE == BWD_DKV ? 22 : 16;
+  constexpr int WSTEP = MODE == BWD_DV ? 1 : MODE == BWD_DKV ? 3 : 2;
   bf16x8 fr[LA];
 #pragma unroll
   for (int i = 0; i < LA; ++i) fr[i] = bf16x8{};
+  floatx4 l4_keep[2] = {zero4, zero4}, d4_keep[2] = {zero4, zero4};
   for (int t = 0; t < n_steps; ++t) {
-    tile_barrier<0>();  // the tiles of steps t and t+1 have landed for everybody; nobody reads that of t-1
-    if (t + 2 < n_steps) {
+    // the tiles of steps t and t+1 have landed for everybody; nobody reads that of t-1
+    if (DEEP && fresh) tile_barrier<DEEP_REQUESTS>();
+    else tile_barrier<0>();
+    if (DEEP) {
+      fresh = t + 3 < n_steps;
+      if (fresh) {
+        load_tile(ld, slot3);
+        load_scalars(ld, slot3);
+        advance(ld);
+      }
+    } else if (t + 2 < n_steps) {
       load_tile(ld, slot2);
       fetch_scalars(ld);
       advance(ld);
@@ -359,6 +460,14 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
       // element pair u are formed in slot WS + WSTEP * u, after dP has drained and before the
       // accumulation needs them.  sched_barrier keeps the compiler from regrouping the slots.
       auto fetch = [&](int f) {
+        if (MODE == BWD_DKV) {
+          const int here = blk * FBLOCK32;  // the block inside the step's slot
+          if (f < 8) return kread_b(kb0, here + FTILE, f);   // dO rows: dP
+          if (f < 16) return vread_b(here + FTILE, f - 8);   // dO^T: dV accumulation
+          if (f < 24) return blk == 0 ? kread_b(kb0, FBLOCK32, f - 16) : kread_b(kb1, 0, f - 16);  // Q rows of the next block: its scores
+          if (f < 32) return vread_b(here, f - 24);          // Q^T: dK accumulation
+          return blk == 0 ? kread_b(kb0, FBLOCK32 + FTILE, f - 32) : kread_b(kb1, FTILE, f - 32);
+        }
         if (MODE == BWD_DV) {
           if (f < 8) return kread(c1n, f);
           if (f < 16) return vread(c2off, f - 8);
@@ -369,12 +478,32 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
         if (f < 24) return vread(c1off, f - 16);
         return kread(c2n, f - 24);
       };
+      const float* sc = DEEP ? reinterpret_cast<const float*>(smem + (sb0 + 128 * blk))
+                             : reinterpret_cast<const float*>(smem + slot0 + 2 * FTILE) + 32 * blk + 4 * g4;
+      // scalars of the block that follows in this order
+      const float* scn = blk == 0 ? sc + 32 : reinterpret_cast<const float*>(smem + sb1);
       if (!have) {  // first block of a run: nothing was prepared by a previous block
-        scores(c1off, s_cur);
+        if (MODE == BWD_DKV) {
+          l4_keep[0] = *reinterpret_cast<const floatx4*>(sc);
+          l4_keep[1] = *reinterpret_cast<const floatx4*>(sc + 16);
+          d4_keep[0] = *reinterpret_cast<const floatx4*>(sc + 64);
+          d4_keep[1] = *reinterpret_cast<const floatx4*>(sc + 64 + 16);
+        }
+        if (DEEP) {
+#pragma unroll
+          for (int t4 = 0; t4 < 4; ++t4) s_cur[t4 >> 1][t4 & 1] = zero4;
+#pragma unroll
+          for (int f = 0; f < 8; ++f) {
+            const bf16x8 a = kread_b(kb0, blk * FBLOCK32, f);
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) s_cur[f & 1][rt] = mfma(a, r1f[rt][f >> 1], s_cur[f & 1][rt]);
+          }
+        } else {
+          scores(c1off, s_cur);
+        }
 #pragma unroll
         for (int i = 0; i < LA; ++i) fr[i] = fetch(i);
       }
-      const float* sc = reinterpret_cast<const float*>(smem + slot0 + 2 * FTILE) + 32 * blk + 4 * g4;
       if (masked) {  // scores of invisible pairs become -inf (for a positive scale): weight 0
 #pragma unroll
         for (int ct = 0; ct < 2; ++ct)
@@ -389,7 +518,12 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
       }
       floatx4 dp[2][2], s_next[2][2];
       bf16x8 wp[2];
-      floatx4 l4[2], d4[2];  // column scalars of the lane's columns, per column tile
+      bf16x8 wp_p[MODE == BWD_DKV ? 2 : 1];   // BWD_DKV: the weights P (wp holds dS)
+      floatx4 pf[MODE == BWD_DKV ? 2 : 1][2];  // BWD_DKV: P before rounding, for dS
+      floatx4 l4_[2], d4_[2];  // column scalars of the lane's columns, per column tile
+      // (BWD_DKV keeps them across blocks: a block reads those of the next one in its last slots)
+      floatx4 (&l4)[2] = MODE == BWD_DKV ? l4_keep : l4_;
+      floatx4 (&d4)[2] = MODE == BWD_DKV ? d4_keep : d4_;
       // weights of pair u = 4 * rt + 2 * ct + h (columns 16 * ct + 4 * g4 + 2 * h, + 1 of row tile rt): P, or dS = P * (dP - D)
       auto stage = [&](int u) {
         const int rt = u >> 2, ct = (u >> 1) & 1, h = u & 1;
@@ -399,20 +533,41 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
           const int e = 2 * h + v;
           const float l = ROWS_ARE_QUERIES ? L2_row[rt] : l4[ct][e];
           float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][rt][e], c2, -l));
-          if (MODE != BWD_DV) x *= dp[ct][rt][e] - (ROWS_ARE_QUERIES ? D_row[rt] : d4[ct][e]);
+          if (MODE != BWD_DV && MODE != BWD_DKV) x *= ROWS_ARE_QUERIES ? dp[ct][rt][e] - D_row[rt] : dp[ct][rt][e] + d4[ct][e];
           w[v] = x;
         }
         floatx2 f2 = {w[0], w[1]};
+        bf16x2 h2 = __builtin_convertvector(f2, bf16x2);
+        if (MODE == BWD_DKV) {  // (this is the P stage: keep the unrounded values for dS)
+          pf[ct][rt][2 * h] = w[0];
+          pf[ct][rt][2 * h + 1] = w[1];
+          wp_p[rt][4 * ct + 2 * h] = h2[0];
+          wp_p[rt][4 * ct + 2 * h + 1] = h2[1];
+        } else {
+          wp[rt][4 * ct + 2 * h] = h2[0];
+          wp[rt][4 * ct + 2 * h + 1] = h2[1];
+        }
+      };
+      // BWD_DKV: dS = P * (dP - D) of pair u; the accumulators of dP start from -D
+      auto stage_ds = [&](int u) {
+        const int rt = u >> 2, ct = (u >> 1) & 1, h = u & 1;
+        floatx2 f2 = {pf[ct][rt][2 * h] * dp[ct][rt][2 * h], pf[ct][rt][2 * h + 1] * dp[ct][rt][2 * h + 1]};  // (dP started from -D)
         bf16x2 h2 = __builtin_convertvector(f2, bf16x2);
         wp[rt][4 * ct + 2 * h] = h2[0];
         wp[rt][4 * ct + 2 * h + 1] = h2[1];
       };
       constexpr int NSLOT = 2 * NFRAG;
-#pragma unroll
-      for (int i = 0; i < NSLOT; ++i) {
-        const int f = i >> 1, rt = i & 1;
+      // (compile-time slot numbers: a loop of this size is beyond what the compiler unrolls in full)
+      static_for<0, NSLOT>([&](auto slot_c) {
+        constexpr int i = decltype(slot_c)::value;
+        constexpr int f = i >> 1, rt = i & 1;
         const bf16x8 a = fr[f % LA];
-        if (MODE == BWD_DV) {
+        if (MODE == BWD_DKV) {
+          if (f < 8) dp[f & 1][rt] = mfma(a, r2f[rt][f >> 1], f < 2 ? d4[f & 1] : dp[f & 1][rt]);  // from -D of the tile's columns
+          else if (f < 16) acc_v[f - 8][rt] = mfma(a, wp_p[rt], acc_v[f - 8][rt]);
+          else if (f < 24) s_next[f & 1][rt] = mfma(a, r1f[rt][(f - 16) >> 1], f < 18 ? zero4 : s_next[f & 1][rt]);
+          else acc[f - 24][rt] = mfma(a, wp[rt], acc[f - 24][rt]);
+        } else if (MODE == BWD_DV) {
           if (f < 8) s_next[f & 1][rt] = mfma(a, r1f[rt][f >> 1], f < 2 ? zero4 : s_next[f & 1][rt]);
           else acc[f - 8][rt] = mfma(a, wp[rt], acc[f - 8][rt]);
         } else {
@@ -421,6 +576,15 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
           else acc[f - 16][rt] = mfma(a, wp[rt], acc[f - 16][rt]);
         }
         if (rt == 1) fr[f % LA] = fetch(f + LA);
+        if (MODE == BWD_DKV) {  // P in front of the dV accumulation, dS behind dP
+          // the next block's scalars, when this block has used its own for the last time
+          if (i == 50) l4[0] = *reinterpret_cast<const floatx4*>(scn);
+          if (i == 52) l4[1] = *reinterpret_cast<const floatx4*>(scn + 16);
+          if (i == 54) d4[0] = *reinterpret_cast<const floatx4*>(scn + 64);
+          if (i == 56) d4[1] = *reinterpret_cast<const floatx4*>(scn + 64 + 16);
+          if (i >= 5 && i < 16 && (i - 5) % 3 != 2) stage((i - 5) - (i - 5) / 3);  // slots 5, 6, 8, 9, 11, 12, 14, 15
+          if (i >= WS && (i - WS) % WSTEP == 0 && (i - WS) / WSTEP < 8) stage_ds((i - WS) / WSTEP);
+        } else {
         if (!ROWS_ARE_QUERIES) {  // column scalars, four slots ahead of the first weight stage
           if (i == WS - 4) l4[0] = *reinterpret_cast<const floatx4*>(sc);
           if (i == WS - 3) l4[1] = *reinterpret_cast<const floatx4*>(sc + 16);
@@ -428,8 +592,9 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
           if (MODE == BWD_DK && i == WS - 1) d4[1] = *reinterpret_cast<const floatx4*>(sc + 64 + 16);
         }
         if (i >= WS && (i - WS) % WSTEP == 0 && (i - WS) / WSTEP < 8) stage((i - WS) / WSTEP);
+        }
         __builtin_amdgcn_sched_barrier(0);
-      }
+      });
 #pragma unroll
       for (int t4 = 0; t4 < 4; ++t4) s_cur[t4 >> 1][t4 & 1] = s_next[t4 >> 1][t4 & 1];
       have = true;
@@ -439,7 +604,24 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
     const int ts = slot0;
     slot0 = slot1;
     slot1 = slot2;
-    slot2 = ts;
+    if (DEEP) {
+      const int d0 = slot0 - ts, d1 = slot1 - slot0;  // (slot0 and slot1 are the new ones already; ts the old slot0)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        kb0[i] += d0;
+        vb0[i] += d0;
+        kb1[i] += d1;
+        // (opaque to the compiler, which would otherwise keep the lane parts and add the slot at every read)
+        asm volatile("" : "+v"(kb0[i]), "+v"(vb0[i]), "+v"(kb1[i]));
+      }
+      sb0 += d0;
+      sb1 += d1;
+      asm volatile("" : "+v"(sb0), "+v"(sb1));
+      slot2 = slot3;
+      slot3 = ts;
+    } else {
+      slot2 = ts;
+    }
   }
 
   // ---------------------------------------------------------------- scale, round, store
@@ -459,40 +641,48 @@ __global__ __launch_bounds__(512) void intra_bwd_kernel(const BParams p) {
   // The four lanes of a row hold head dims 4 * g4 .. + 3 of every 16-dim tile; a lane quarter and
   // its neighbour trade 8 bytes per tile pair so that each lane owns the whole 16-byte chunk
   // 4 * m + 2 * (g4 % 2) + g4 / 2 of its row.
+  auto store_rows = [&](const floatx4 (&a)[8][2], int what, float factor) {
 #pragma unroll
-  for (int rt = 0; rt < 2; ++rt) {
-    const bool keep = row_valid[rt] && map.store((int)rpos[rt]);
-    uint16_t* orow;
-    const int cofs = (2 * (g4 & 1) + (g4 >> 1)) * 8;
-    if (MODE == BWD_DQ) orow = p.dq + (batch * p.dq_bs + rpos[rt] * p.dq_rs + hq * p.dq_hs + cofs);
-    else if (MODE == BWD_DK) orow = p.dk + (batch * p.dk_bs + rpos[rt] * p.dk_rs + kvh * p.dk_hs + cofs);
-    else orow = p.dv + (batch * p.dv_bs + rpos[rt] * p.dv_rs + kvh * p.dv_hs + cofs);
+    for (int rt = 0; rt < 2; ++rt) {
+      const bool keep = row_valid[rt] && map.store((int)rpos[rt]);
+      uint16_t* orow;
+      const int cofs = (2 * (g4 & 1) + (g4 >> 1)) * 8;
+      if (what == BWD_DQ) orow = p.dq + (batch * p.dq_bs + rpos[rt] * p.dq_rs + hq * p.dq_hs + cofs);
+      else if (what == BWD_DK) orow = p.dk + (batch * p.dk_bs + rpos[rt] * p.dk_rs + kvh * p.dk_hs + cofs);
+      else orow = p.dv + (batch * p.dv_bs + rpos[rt] * p.dv_rs + kvh * p.dv_hs + cofs);
 #pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      uint32_t w[2][2];
+      for (int m = 0; m < 4; ++m) {
+        uint32_t w[2][2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int k2 = 0; k2 < 2; ++k2) {
-          floatx2 v2 = {acc[2 * m + t][rt][2 * k2] * f, acc[2 * m + t][rt][2 * k2 + 1] * f};
-          w[t][k2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
-        }
-      auto q0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
-      auto q1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
-      if (keep) {
-        u32x4 pk = {q0[0], q1[0], q0[1], q1[1]};
-        if (RMAP::kAccumulate) {  // add to what an earlier pass has written (both rounded to bf16)
-          const u32x4 old = *reinterpret_cast<const u32x4*>(orow + 32 * m);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            floatx2 s2 = {__uint_as_float(pk[i] << 16) + __uint_as_float(old[i] << 16),
-                          __uint_as_float(pk[i] & 0xffff0000u) + __uint_as_float(old[i] & 0xffff0000u)};
-            pk[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(s2, bf16x2));
+          for (int k2 = 0; k2 < 2; ++k2) {
+            floatx2 v2 = {a[2 * m + t][rt][2 * k2] * factor, a[2 * m + t][rt][2 * k2 + 1] * factor};
+            w[t][k2] = __builtin_bit_cast(uint32_t, __builtin_convertvector(v2, bf16x2));
           }
+        auto q0 = __builtin_amdgcn_permlane16_swap(w[0][0], w[1][0], false, false);
+        auto q1 = __builtin_amdgcn_permlane16_swap(w[0][1], w[1][1], false, false);
+        if (keep) {
+          u32x4 pk = {q0[0], q1[0], q0[1], q1[1]};
+          if (RMAP::kAccumulate) {  // add to what an earlier pass has written (both rounded to bf16)
+            const u32x4 old = *reinterpret_cast<const u32x4*>(orow + 32 * m);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              floatx2 s2 = {__uint_as_float(pk[i] << 16) + __uint_as_float(old[i] << 16),
+                            __uint_as_float(pk[i] & 0xffff0000u) + __uint_as_float(old[i] & 0xffff0000u)};
+              pk[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(s2, bf16x2));
+            }
+          }
+          *reinterpret_cast<u32x4*>(orow + 32 * m) = pk;
         }
-        *reinterpret_cast<u32x4*>(orow + 32 * m) = pk;
       }
     }
+  };
+  if constexpr (MODE == BWD_DKV) {
+    store_rows(acc, BWD_DK, p.scale);
+    store_rows(acc_v, BWD_DV, 1.f);
+  } else {
+    store_rows(acc, MODE, f);
   }
 }
 

@@ -308,18 +308,19 @@ def _leading_chunks(S, B, Hkv, ns, cus=320):
 
 
 def test_bwd_workspace_size(lib):
-    assert lib.intra_llm_bwd_workspace(1, 1000, 8, 2, 0, 8, 576, 256, 0, 0) == 8000
-    assert lib.intra_llm_bwd_workspace(2, 1001, 3, 3, 4, 8, 576, 256, 0, 0) == 6008  # rounded up to 4
+    # two values per (batch, head, token): -rowsum(dO o O) and lse * log2(e)
+    assert lib.intra_llm_bwd_workspace(1, 1000, 8, 2, 0, 8, 576, 256, 0, 0) == 2 * 8000
+    assert lib.intra_llm_bwd_workspace(2, 1001, 3, 3, 4, 8, 576, 256, 0, 0) == 2 * 6008  # each rounded up to 4
     # sinks: chunks x B x Hkv x n_sink x 128 more
     assert _leading_chunks(3000, 1, 2, 64) == 16 and _leading_chunks(65536, 1, 8, 64) == 40
-    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 24000 + 16 * 2 * 64 * 128
-    assert lib.intra_llm_bwd_workspace(1, 65536, 32, 8, 9, 2, 575, 256, 0, 64) == 65536 * 32 + 40 * 8 * 64 * 128
-    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 256, 1, 0) == 24000
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 9, 2, 575, 256, 0, 64) == 2 * 24000 + 16 * 2 * 64 * 128
+    assert lib.intra_llm_bwd_workspace(1, 65536, 32, 8, 9, 2, 575, 256, 0, 64) == 2 * 65536 * 32 + 40 * 8 * 64 * 128
+    assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 256, 1, 0) == 2 * 24000
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 2, 8, 2, 575, 128, 1, 0) == -1
     assert lib.intra_llm_bwd_workspace(1, 3000, 8, 3, 0, 8, 576, 256, 0, 0) == -1
     # image patterns: the 512 text keys are the leading keys
     S = 512 + 64 * 64
-    assert lib.intra_image_bwd_workspace(1, S, 24, 24, 0, 64, 512) == S * 24 + _leading_chunks(S, 1, 24, 512) * 24 * 512 * 128
+    assert lib.intra_image_bwd_workspace(1, S, 24, 24, 0, 64, 512) == 2 * S * 24 + _leading_chunks(S, 1, 24, 512) * 24 * 512 * 128
     assert lib.intra_image_bwd_workspace(1, S, 24, 24, 4, 64, 511) == -1
 
 
