@@ -256,6 +256,25 @@ DIAG_SLOTS = 16  # values per workgroup (csrc/intra_kernel.hip.h)
 BARRIERS = ["in front of the Q slots", "in front of the first key block", "opening tile 0", "between tiles (per tile)"]
 
 
+def placement(raw, iters):
+    """Half-size workgroups: which share a CU, and the busy time of the one in the CU's first wavefront
+    slot against the one in its second (HW_ID of wavefront 0, written over - not added to - slot 8)."""
+    raw = raw[raw[:, 5] > 0]
+    hw = raw[:, 8]
+    cu = (((hw >> 32) & 0xF) << 12) | (((hw >> 13) & 7) << 8) | (((hw >> 12) & 1) << 4) | ((hw >> 8) & 0xF)  # XCC, SE, SH, CU
+    slot = hw & 0xF
+    busy = raw[:, :5].sum(1).double() / 100 / iters
+    per_cu = {}
+    for i in range(raw.shape[0]):
+        per_cu.setdefault(int(cu[i]), []).append(i)
+    sizes = sorted({len(v) for v in per_cu.values()})
+    first = [busy[i].item() for v in per_cu.values() for i in v if slot[i] == 0]
+    second = [busy[i].item() for v in per_cu.values() for i in v if slot[i] != 0]
+    return {"cus": len(per_cu), "workgroups_per_cu": sizes,
+            "busy_us_first_slot": round(sum(first) / max(1, len(first)), 1),
+            "busy_us_second_slot": round(sum(second) / max(1, len(second)), 1)}
+
+
 @torch.no_grad()
 def bench_phases(args):
     """Sum over a launch of the in-kernel phase timers (see include/intra_hip.h, intra_diag_set_buffer)."""
@@ -298,10 +317,15 @@ def bench_phases(args):
     res["share_outside_tile_loop"] = round(1 - d[:, 3].sum().item() / d[:, :5].sum().item(), 4)
     # shader cycles -> us with the clock of the tile loops; [own requests and LDS reads, other wavefronts]
     mhz = d[:, 7].mean().item() / loop_us
+    res["waves"] = 4 if d.shape[0] > torch.cuda.get_device_properties(0).multi_processor_count else 8
     res["barrier_wait_us"] = {}
     for i, name in enumerate(BARRIERS):
+        if res["waves"] == 4 and i < 3:
+            continue  # half-size workgroups have no barriers at the item boundary (slots 8 .. 11 hold the placement)
         per = tiles if i == 3 else items
         res["barrier_wait_us"][name] = [round(d[:, 8 + 2 * i + j].mean().item() / mhz / per, 3) for j in range(2)]
+    if res["waves"] == 4:
+        res["placement"] = placement(buf.view(-1, DIAG_SLOTS).cpu(), args.iters)
     print(json.dumps(res), flush=True)
     return [res]
 
