@@ -10,6 +10,10 @@
  * default of the softmax arithmetic (intra_set_softmax_mode; a call can name its own in the flags
  * of the *_ex entry points), the 16 MiB per-GPU array behind intra_llm_bwd_noalloc, the timer buffer
  * of measurement builds (intra_diag_set_buffer), and per-device caches of the CU count.
+ * Environment variables read by the library, both for experiments only: INTRA_SOFTMAX (the
+ * starting value of that default) and INTRA_WAVES (8 or 4: the workgroup size of the forward
+ * launches, where the named shape exists; otherwise the library picks - workgroups of 4 wavefronts,
+ * two per CU, for image gather0 and for launches with few row blocks, 8 wavefronts for the rest).
  *
  * Every function returns INTRA_OK or an error code; intra_last_error() then describes the failure
  * (thread-local string).  Argument validation happens before any HIP call, so it can be exercised
@@ -256,7 +260,8 @@ int intra_model_mask(int domain, int pattern, int S, int arg0, int arg1, int hea
 int intra_model_deal(int domain, int pattern, int B, int S, int H, int Hkv, int arg0, int arg1,
                      int waves, int grid, uint8_t* visits, int64_t n_visits);
 
-/* intra_plan / intra_model_mask for the arguments of intra_llm_fwd_ex (always 8 wavefronts). */
+/* intra_plan / intra_model_mask for the arguments of intra_llm_fwd_ex (the walk: row blocks of 8
+ * wavefronts). */
 int intra_plan_llm_ex(int pattern, int B, int S, int H, int Hkv, int group_num, int window,
                       int block, int offset, int n_sink, IntraPlan* plan);
 int intra_model_mask_llm_ex(int pattern, int S, int group_num, int window, int block, int offset,
@@ -280,7 +285,10 @@ int intra_model_mask_image_bwd(int pattern, int S, int width, int text_len, uint
  * [4] look-up of the next item, its Q request, normalisation and stores; [5] work items, [6] key
  * tiles, [7] shader cycles of the tile loops; [8]..[15] shader cycles at the barriers in front of
  * the Q slots, of the first key block, of tile 0 and between tiles, each as a pair {waiting for the
- * wavefront's own requests and LDS reads, waiting for the other wavefronts}.  NULL switches it off.  A production build returns
+ * wavefront's own requests and LDS reads, waiting for the other wavefronts}.  Launches of workgroups
+ * of 4 wavefronts have no barriers at the item boundary: [1] stays 0, and [8]..[11] are WRITTEN with
+ * the hardware id of wavefronts 0..3 (HW_ID register in the low half, XCC_ID above it), from which a
+ * reader sees which workgroups share a CU.  NULL switches it off.  A production build returns
  * INTRA_ERR_UNSUPPORTED and never touches such a buffer.
  *
  * intra_diag_mfma_ceiling: one launch of `workgroups` x 8 wavefronts that issue nothing but bf16
