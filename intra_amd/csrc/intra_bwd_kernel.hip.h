@@ -411,6 +411,8 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
 #pragma unroll
   for (int i = 0; i < LA; ++i) fr[i] = bf16x8{};
   floatx4 l4_keep[2] = {zero4, zero4}, d4_keep[2] = {zero4, zero4};
+  // dQ: -D of the lane's two rows, as the accumulators of dP start from it
+  const floatx4 nd_row[2] = {floatx4{-D_row[0], -D_row[0], -D_row[0], -D_row[0]}, floatx4{-D_row[1], -D_row[1], -D_row[1], -D_row[1]}};
   for (int t = 0; t < n_steps; ++t) {
     // the tiles of steps t and t+1 have landed for everybody; nobody reads that of t-1
     if (DEEP && fresh) tile_barrier<DEEP_REQUESTS>();
@@ -533,7 +535,7 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
           const int e = 2 * h + v;
           const float l = ROWS_ARE_QUERIES ? L2_row[rt] : l4[ct][e];
           float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][rt][e], c2, -l));
-          if (MODE != BWD_DV && MODE != BWD_DKV) x *= ROWS_ARE_QUERIES ? dp[ct][rt][e] - D_row[rt] : dp[ct][rt][e] + d4[ct][e];
+          if (MODE != BWD_DV && MODE != BWD_DKV) x *= ROWS_ARE_QUERIES ? dp[ct][rt][e] : dp[ct][rt][e] + d4[ct][e];  // (dQ: dP started from -D)
           w[v] = x;
         }
         floatx2 f2 = {w[0], w[1]};
@@ -571,7 +573,7 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
           if (f < 8) s_next[f & 1][rt] = mfma(a, r1f[rt][f >> 1], f < 2 ? zero4 : s_next[f & 1][rt]);
           else acc[f - 8][rt] = mfma(a, wp[rt], acc[f - 8][rt]);
         } else {
-          if (f < 8) dp[f & 1][rt] = mfma(a, r2f[rt][f >> 1], f < 2 ? zero4 : dp[f & 1][rt]);
+          if (f < 8) dp[f & 1][rt] = mfma(a, r2f[rt][f >> 1], f < 2 ? (ROWS_ARE_QUERIES ? nd_row[rt] : zero4) : dp[f & 1][rt]);  // dQ: from -D of the row
           else if (f < 16) s_next[f & 1][rt] = mfma(a, r1f[rt][(f - 8) >> 1], f < 10 ? zero4 : s_next[f & 1][rt]);
           else acc[f - 16][rt] = mfma(a, wp[rt], acc[f - 16][rt]);
         }
