@@ -90,6 +90,7 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
   // its ring is one slot deeper and a tile has two steps to land; the column scalars travel the same
   // way (every wavefront requests those of 16 columns) instead of through registers.
   constexpr bool DEEP = MODE == BWD_DKV;
+  constexpr bool TWO_STAGES = MODE == BWD_DKV || MODE == BWD_DQ;  // P and dS = P * dP formed apart
   __shared__ __attribute__((aligned(1024))) unsigned char smem[bwd_ring_slots(MODE) * BWD_SLOT];
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
@@ -230,20 +231,11 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
     for (int a = 0; a < 4; ++a)
       vaddr[a] = g4 * FGROUP_STRIDE + ri * 256 + 64 * (a ^ ri) + 16 * ((l16 & 3) >> 1) + 8 * (l16 & 1);
   }
-  // row-per-lane operand 2 * ks + ct of a 32-row block: rows 16 * ct + l16, head dims of k-step ks
-  auto kread = [&](int off, int f) {
-    return *reinterpret_cast<const bf16x8*>(smem + off + kaddr[f >> 1] + (f & 1) * 4 * FGROUP_STRIDE);
-  };
-  // transposed operand: head dims 16 * dt .. + 15 of the block's 32 rows
-  auto vread = [&](int off, int dt) {
-    const int o2 = off + vaddr[dt >> 1] + 32 * (dt & 1);
-    bf16x4 v0 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((__attribute__((address_space(3))) bf16x4*)(smem + o2));
-    bf16x4 v1 = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-        (__attribute__((address_space(3))) bf16x4*)(smem + o2 + 4 * FGROUP_STRIDE));
-    return __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
-  };
-  // Deep ring: the same reads from per-lane bases that carry the ring slot (b0: the step's slot, b1:
-  // the next one's), advanced once per step, so that everything else is a compile-time offset
+  // LDS operands are read from per-lane bases that carry the ring slot (b0: the step's slot, b1: the
+  // next one's), advanced once per step, so that everything else is a compile-time offset.
+  // kread_b: row-per-lane operand 2 * ks + ct of a 32-row block (rows 16 * ct + l16, head dims of
+  // k-step ks); vread_b: transposed operand (head dims 16 * dt .. + 15 of the block's 32 rows).
+  // sb0, sb1: the same for the column scalars of the deep ring.
   int kb0[4], kb1[4], vb0[4], sb0 = 0, sb1 = 0;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -360,18 +352,6 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
       sc[64 + lane] = sc_d;
     }
   };
-  // scores of a block whose rows start at LDS offset `off`, outside the schedule
-  auto scores = [&](int off, floatx4 (&s)[2][2]) {
-#pragma unroll
-    for (int t = 0; t < 4; ++t) s[t >> 1][t & 1] = zero4;
-#pragma unroll
-    for (int f = 0; f < 8; ++f) {
-      const bf16x8 a = kread(off, f);
-#pragma unroll
-      for (int rt = 0; rt < 2; ++rt) s[f & 1][rt] = mfma(a, r1f[rt][f >> 1], s[f & 1][rt]);
-    }
-  };
-
   // Three tile slots: while step t works on its tile, the tile of step t+1 has landed (the scores
   // of its first block are formed at the end of step t) and the tile of step t+2 is in flight.
   Cursor cur{ROWS_ARE_QUERIES ? 0 : ntiles - 1, 0};  // step being computed
@@ -451,10 +431,6 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
       } else {
         masked = !block_unmasked(wb, kpre, sb_lo);
       }
-      // this block, the one that follows in this order, and the one after that
-      const int c1off = slot0 + blk * FBLOCK32, c2off = c1off + FTILE;
-      const int c1n = blk == 0 ? c1off + FBLOCK32 : slot1, c2n = c1n + FTILE;
-      const int c1nn = blk == 0 ? slot1 : slot1 + FBLOCK32;
       // Hand-scheduled.  dQ / dK: slots 0-15 dP of this block, 16-31 the scores of the next block,
       // 32-47 the accumulation; dV: 0-15 scores of the next block, 16-31 the accumulation.  LDS
       // operand f (slots 2f, 2f+1) is requested LA operands earlier into a ring of LA fragments,
@@ -462,23 +438,27 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
       // element pair u are formed in slot WS + WSTEP * u, after dP has drained and before the
       // accumulation needs them.  sched_barrier keeps the compiler from regrouping the slots.
       auto fetch = [&](int f) {
+        const int here = blk * FBLOCK32;  // the block inside the step's slot
+        // rows of the block that follows in this order, at tile `which` of its slot
+        auto next_rows = [&](int which, int ff) {
+          return blk == 0 ? kread_b(kb0, FBLOCK32 + which * FTILE, ff) : kread_b(kb1, which * FTILE, ff);
+        };
         if (MODE == BWD_DKV) {
-          const int here = blk * FBLOCK32;  // the block inside the step's slot
           if (f < 8) return kread_b(kb0, here + FTILE, f);   // dO rows: dP
           if (f < 16) return vread_b(here + FTILE, f - 8);   // dO^T: dV accumulation
-          if (f < 24) return blk == 0 ? kread_b(kb0, FBLOCK32, f - 16) : kread_b(kb1, 0, f - 16);  // Q rows of the next block: its scores
+          if (f < 24) return next_rows(0, f - 16);           // Q rows of the next block: its scores
           if (f < 32) return vread_b(here, f - 24);          // Q^T: dK accumulation
-          return blk == 0 ? kread_b(kb0, FBLOCK32 + FTILE, f - 32) : kread_b(kb1, FTILE, f - 32);
+          return next_rows(1, f - 32);
         }
         if (MODE == BWD_DV) {
-          if (f < 8) return kread(c1n, f);
-          if (f < 16) return vread(c2off, f - 8);
-          return kread(c1nn, f - 16);
+          if (f < 8) return next_rows(0, f);
+          if (f < 16) return vread_b(here + FTILE, f - 8);
+          return blk == 0 ? kread_b(kb1, 0, f - 16) : kread_b(kb1, FBLOCK32, f - 16);  // the block after the next
         }
-        if (f < 8) return kread(c2off, f);
-        if (f < 16) return kread(c1n, f - 8);
-        if (f < 24) return vread(c1off, f - 16);
-        return kread(c2n, f - 24);
+        if (f < 8) return kread_b(kb0, here + FTILE, f);
+        if (f < 16) return next_rows(0, f - 8);
+        if (f < 24) return vread_b(here, f - 16);
+        return next_rows(1, f - 24);
       };
       const float* sc = DEEP ? reinterpret_cast<const float*>(smem + (sb0 + 128 * blk))
                              : reinterpret_cast<const float*>(smem + slot0 + 2 * FTILE) + 32 * blk + 4 * g4;
@@ -491,17 +471,13 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
           d4_keep[0] = *reinterpret_cast<const floatx4*>(sc + 64);
           d4_keep[1] = *reinterpret_cast<const floatx4*>(sc + 64 + 16);
         }
-        if (DEEP) {
 #pragma unroll
-          for (int t4 = 0; t4 < 4; ++t4) s_cur[t4 >> 1][t4 & 1] = zero4;
+        for (int t4 = 0; t4 < 4; ++t4) s_cur[t4 >> 1][t4 & 1] = zero4;
 #pragma unroll
-          for (int f = 0; f < 8; ++f) {
-            const bf16x8 a = kread_b(kb0, blk * FBLOCK32, f);
+        for (int f = 0; f < 8; ++f) {
+          const bf16x8 a = kread_b(kb0, blk * FBLOCK32, f);
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) s_cur[f & 1][rt] = mfma(a, r1f[rt][f >> 1], s_cur[f & 1][rt]);
-          }
-        } else {
-          scores(c1off, s_cur);
+          for (int rt = 0; rt < 2; ++rt) s_cur[f & 1][rt] = mfma(a, r1f[rt][f >> 1], s_cur[f & 1][rt]);
         }
 #pragma unroll
         for (int i = 0; i < LA; ++i) fr[i] = fetch(i);
@@ -521,7 +497,7 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
       floatx4 dp[2][2], s_next[2][2];
       bf16x8 wp[2];
       bf16x8 wp_p[MODE == BWD_DKV ? 2 : 1];   // BWD_DKV: the weights P (wp holds dS)
-      floatx4 pf[MODE == BWD_DKV ? 2 : 1][2];  // BWD_DKV: P before rounding, for dS
+      floatx4 pf[TWO_STAGES ? 2 : 1][2];       // P before rounding, for dS
       floatx4 l4_[2], d4_[2];  // column scalars of the lane's columns, per column tile
       // (BWD_DKV keeps them across blocks: a block reads those of the next one in its last slots)
       floatx4 (&l4)[2] = MODE == BWD_DKV ? l4_keep : l4_;
@@ -535,8 +511,13 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
           const int e = 2 * h + v;
           const float l = ROWS_ARE_QUERIES ? L2_row[rt] : l4[ct][e];
           float x = __builtin_amdgcn_exp2f(__builtin_fmaf(s_cur[ct][rt][e], c2, -l));
-          if (MODE != BWD_DV && MODE != BWD_DKV) x *= ROWS_ARE_QUERIES ? dp[ct][rt][e] : dp[ct][rt][e] + d4[ct][e];  // (dQ: dP started from -D)
+          if (MODE == BWD_DK) x *= dp[ct][rt][e] + d4[ct][e];
           w[v] = x;
+        }
+        if (MODE == BWD_DQ) {  // (the P stage: dS follows when dP is there)
+          pf[ct][rt][2 * h] = w[0];
+          pf[ct][rt][2 * h + 1] = w[1];
+          return;
         }
         floatx2 f2 = {w[0], w[1]};
         bf16x2 h2 = __builtin_convertvector(f2, bf16x2);
@@ -550,7 +531,7 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
           wp[rt][4 * ct + 2 * h + 1] = h2[1];
         }
       };
-      // BWD_DKV: dS = P * (dP - D) of pair u; the accumulators of dP start from -D
+      // dQ and BWD_DKV: dS = P * (dP - D) of pair u; the accumulators of dP start from -D
       auto stage_ds = [&](int u) {
         const int rt = u >> 2, ct = (u >> 1) & 1, h = u & 1;
         floatx2 f2 = {pf[ct][rt][2 * h] * dp[ct][rt][2 * h], pf[ct][rt][2 * h + 1] * dp[ct][rt][2 * h + 1]};  // (dP started from -D)
@@ -593,7 +574,12 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
           if (MODE == BWD_DK && i == WS - 2) d4[0] = *reinterpret_cast<const floatx4*>(sc + 64);
           if (MODE == BWD_DK && i == WS - 1) d4[1] = *reinterpret_cast<const floatx4*>(sc + 64 + 16);
         }
-        if (i >= WS && (i - WS) % WSTEP == 0 && (i - WS) / WSTEP < 8) stage((i - WS) / WSTEP);
+        // dQ: P while dP is formed (the scores are then free for those of the next block), dS behind it
+        if (MODE == BWD_DQ && i < 16 && i % 2 == 0) stage(i / 2);
+        if (i >= WS && (i - WS) % WSTEP == 0 && (i - WS) / WSTEP < 8) {
+          if (MODE == BWD_DQ) stage_ds((i - WS) / WSTEP);
+          else stage((i - WS) / WSTEP);
+        }
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -606,7 +592,7 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
     const int ts = slot0;
     slot0 = slot1;
     slot1 = slot2;
-    if (DEEP) {
+    {
       const int d0 = slot0 - ts, d1 = slot1 - slot0;  // (slot0 and slot1 are the new ones already; ts the old slot0)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -616,9 +602,13 @@ __global__ __launch_bounds__(bwd_waves(MODE) * 64) void intra_bwd_kernel(const B
         // (opaque to the compiler, which would otherwise keep the lane parts and add the slot at every read)
         asm volatile("" : "+v"(kb0[i]), "+v"(vb0[i]), "+v"(kb1[i]));
       }
-      sb0 += d0;
-      sb1 += d1;
-      asm volatile("" : "+v"(sb0), "+v"(sb1));
+      if (DEEP) {
+        sb0 += d0;
+        sb1 += d1;
+        asm volatile("" : "+v"(sb0), "+v"(sb1));
+      }
+    }
+    if (DEEP) {
       slot2 = slot3;
       slot3 = ts;
     } else {
