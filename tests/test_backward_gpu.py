@@ -289,7 +289,7 @@ def _random_cases(n, seed):
     return cases
 
 
-@pytest.mark.parametrize("case", _random_cases(40, seed=77), ids=lambda c: f"{c[0]}-S{c[2]}-H{c[3]}/{c[4]}")
+@pytest.mark.parametrize("case", _random_cases(40, seed=77) + _random_cases(80, seed=78), ids=lambda c: f"{c[0]}-S{c[2]}-H{c[3]}/{c[4]}")
 def test_random_shapes(case):
     kind, B, S, H, Hkv, kw, scale = case
     run_case(f"llm/{kind}", kind, B, S, H, Hkv, seed=S + H, scale=scale, **kw)

@@ -59,6 +59,52 @@ def test_llm_patterns_with_either_size(waves, pattern, kw, S, H, Hkv):
     assert torch.equal(plain, outs[8]) or torch.equal(plain, outs[4])
 
 
+def _random_cases(n, seed):
+    """Random shapes, patterns, head ratios (1 - 8 query heads per kv head) and scales; the arguments
+    stay inside what both workgroup sizes accept (a striped block pattern with an offset needs blocks
+    of 128 tokens per odd head ratio for the half-size kernel, of 256 for the other)."""
+    import random
+    rnd = random.Random(seed)
+    heads = [(4, 4), (4, 2), (8, 2), (4, 1), (16, 4), (3, 3), (6, 3), (32, 8), (5, 1), (12, 2), (2, 2), (1, 1)]
+    cases = []
+    for _ in range(n):
+        H, Hkv = rnd.choice(heads)
+        S = rnd.choice([rnd.randint(1, 300), rnd.randint(300, 3000), 64 * rnd.randint(1, 40), rnd.randint(3000, 6000)])
+        B = 1 if S * H > 48000 else rnd.choice([1, 2, 3])
+        kind = rnd.choice(["scatter", "gather1", "window", "block_scatter", "window_sink"])
+        if kind == "scatter":
+            kw = dict(group_num=rnd.choice([1, 2, 3, 4, 5, 7, 8, 13, 16]))
+        elif kind == "gather1":
+            S = 64 * max(1, S // 64)
+            kw = dict(group_num=8)
+        elif kind == "window":
+            kw = dict(window=rnd.choice([64, 65, 128, 576, 1000, 4000, rnd.randint(64, 3000)]))
+        elif kind == "block_scatter":
+            G = rnd.choice([1, 2, 3, 4])
+            off = rnd.randrange(G)
+            blk = 256 * rnd.choice([1, 1, 2]) if (off or (H // Hkv) % 4) else 64 * rnd.choice([1, 2, 4, 8])
+            kw = dict(group_num=G, block=blk, offset=off, n_sink=rnd.choice([0, 1, 64, blk, rnd.randint(0, blk)]))
+        else:
+            kw = dict(window=rnd.choice([1, 2, 63, 64, 575, 2000, rnd.randint(1, 1500)]),
+                      n_sink=rnd.choice([0, 1, 64, 100, 700, rnd.randint(0, 500)]))
+        cases.append((kind, B, S, H, Hkv, kw, rnd.choice([None, None, 0.05, -0.11, 0.2])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_cases(120, seed=5), ids=lambda c: f"{c[0]}-S{c[2]}-H{c[3]}/{c[4]}")
+def test_random_shapes_with_either_size(waves, case):
+    """Whole outputs and log-sum-exps against the oracle, for a plain call and for each size by name."""
+    kind, B, S, H, Hkv, kw, scale = case
+    q, k, v = make_qkv(B, S, H, Hkv, seed=S + 7 * H)
+    ref = oracle.masked_lse_rows(q, k, oracle.mask_rows(f"llm/{kind}", S, device=DEV, **kw), softmax_scale=scale)
+    for n in (None, 4, 8):
+        waves(n)
+        with torch.no_grad():
+            out, lse = intra_llm_attn(q, k, v, kind, softmax_scale=scale, return_lse=True, **kw)
+        check(out, q, k, v, f"llm/{kind}", None, scale, True, f"{kind} S={S} H={H}/{Hkv} waves={n}", **kw)
+        assert (lse - ref).abs().max().item() <= 5e-3
+
+
 @pytest.mark.parametrize("width", [64, 128])
 @pytest.mark.parametrize("pattern", ["scatter", "gather0"])
 def test_image_patterns_with_either_size(waves, pattern, width):
