@@ -122,6 +122,61 @@ def test_image_patterns_with_either_size(waves, pattern, width):
         assert torch.equal(outs[8], outs[4])
 
 
+def _random_image_cases(n, seed):
+    import random
+    rnd = random.Random(seed)
+    heads = [(4, 4), (4, 2), (8, 2), (4, 1), (3, 3), (6, 3), (24, 24), (5, 1), (2, 2), (1, 1), (6, 1)]
+    cases = []
+    for _ in range(n):
+        H, Hkv = rnd.choice(heads)
+        width = 8 * rnd.choice([2, 3, 4, 5, 6, 7, 8, 8, 9, 10, 12])
+        text_len = 8 * rnd.choice([1, 2, 4, 8, 9, 12, 25, 32, 64, 64, 33, 100])
+        cases.append((rnd.choice([("scatter", 0), ("gather0", 4)]), width, text_len, rnd.choice([1, 2]), H, Hkv,
+                      rnd.choice([128 ** -0.5, 0.05, -0.11])))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_image_cases(40, seed=6), ids=lambda c: f"{c[0][0]}-W{c[1]}-T{c[2]}-H{c[4]}/{c[5]}")
+def test_random_image_shapes_with_either_size_and_their_gradients(waves, case):
+    """Grids of 16 - 96 tokens a side and 8 - 800 text tokens through the C ABI: outputs and
+    log-sum-exps of each size against the oracle, then the backward of the plain call's result."""
+    from test_backward_gpu import compare
+    (pattern, pid), width, text_len, B, H, Hkv, scale = case
+    lib = _lib.load()
+    S = text_len + width * width
+    g = torch.Generator(device="cpu").manual_seed(S + H)
+    mk = lambda h: torch.randn(B, S, h, 128, generator=g, dtype=torch.float32).to(torch.bfloat16).to(DEV)
+    q, k, v, dout = mk(H), mk(Hkv), mk(Hkv), mk(H)
+    stream = torch.cuda.current_stream().cuda_stream
+    mask = oracle.mask_rows(f"image/{pattern}", S, device=DEV, width=width, text_len=text_len)
+    ref_lse = oracle.masked_lse_rows(q, k, mask, softmax_scale=scale)
+    for n in (8, 4, None):
+        waves(n)
+        out = torch.full_like(q, float("nan"))
+        lse = torch.full((B, H, S), float("nan"), dtype=torch.float32, device=DEV)
+        rc = lib.intra_image_fwd_lse(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), B, S, H, Hkv,
+                                     _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out),
+                                     pid, width, text_len, scale, stream, lse.data_ptr(), _lib.strides3(lse))
+        assert rc == 0, _lib.last_error()
+        torch.cuda.synchronize()
+        check(out, q, k, v, f"image/{pattern}", None, scale, True, f"{pattern} W={width} T={text_len} waves={n}",
+              width=width, text_len=text_len)
+        assert (lse - ref_lse).abs().max().item() <= 5e-3
+    nws = lib.intra_image_bwd_workspace(B, S, H, Hkv, pid, width, text_len)
+    work = torch.full((nws + 64,), float("nan"), dtype=torch.float32, device=DEV)
+    dq, dk, dv = (torch.full_like(t, float("nan")) for t in (q, k, v))
+    rc = lib.intra_image_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), lse.data_ptr(), dout.data_ptr(),
+                             dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), work.data_ptr(), B, S, H, Hkv,
+                             _lib.strides3(q), _lib.strides3(k), _lib.strides3(v), _lib.strides3(out), _lib.strides3(dout),
+                             _lib.strides3(dq), _lib.strides3(dk), _lib.strides3(dv), _lib.strides3(lse),
+                             pid, width, text_len, scale, stream)
+    assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(work[nws:]).all()), "wrote past the workspace"
+    compare((dq, dk, dv), oracle.masked_attention_grads(q, k, v, dout, mask, softmax_scale=scale),
+            f"image/{pattern} W={width} T={text_len}")
+
+
 def test_the_plan_names_what_a_plain_call_runs(waves):
     lib = _lib.load()
     plan = _lib.IntraPlan()
